@@ -1,0 +1,572 @@
+// Sequence-mixer kernels for stateful / latent-cache decoder layers (gfx950, wave64).
+//
+// One ragged step is [tokens of sequence 0 | tokens of sequence 1 | ...]; a sequence is
+// described by qsl[s] (first row), seq_lens[s] (tokens held after this step) and
+// slots[s] (its row in every per-sequence state tensor, < 0 = padding row). A sequence
+// whose context is empty (seq_len == q_len) starts from zero state whatever its slot
+// holds, so a slot needs no clearing when it is handed to another request.
+//
+//   embed_rows          token ids -> fp32 residual rows
+//   canon_conv          h + causal depthwise conv over time, carried by [taps-1] rows of state
+//   scaled_add_rmsnorm  x <- rmsnorm(alpha * x + y + bias) * (offset + w)   (fp32 residual)
+//   latent_prep         query latent norm; key/value latent norm + rotated shared key -> paged latent cache
+//   latent_attention    windowed softmax attention in latent space (all heads share the cached rows)
+//   delta_scan          S <- diag(w) S - (a u)(u^T S) + k v^T ; o = S^T r   (fp32 state per slot)
+//   delta_out           per-head unit-rms, weight and sigmoid gate
+//   xielu, tanh_cols    activations
+//
+// Activations / caches are T = float or bf16 (raw uint16_t); everything the recurrences,
+// norms, softmax and rotations touch is fp32.
+#include "common.h"
+
+#include <algorithm>
+
+namespace xgm {
+using xgk::bf2f;
+using xgk::block_sum;
+using xgk::f2bf;
+using xgk::wave_max;
+using xgk::wave_sum;
+typedef uint16_t bf16;
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p);
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ldf<bf16>(const bf16* p) { return bf2f(*p); }
+template <typename T> __device__ __forceinline__ void stf(T* p, float v);
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void stf<bf16>(bf16* p, float v) { *p = f2bf(v); }
+
+__device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + expf(-x)); }
+
+// ------------------------------------------------------------------ embedding
+template <typename TW>
+__global__ void embed_rows_kernel(const int32_t* __restrict__ ids, const TW* __restrict__ table, float* __restrict__ out,
+                                  int W, int V) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  const bool ok = id >= 0 && id < V;
+  for (int c = threadIdx.x; c < W; c += blockDim.x)
+    out[(int64_t)t * W + c] = ok ? ldf(table + (int64_t)id * W + c) : 0.f;
+}
+
+// ------------------------------------------------------------------ causal conv with carried inputs
+constexpr int kMaxTaps = 8;
+
+// state[slot][k][c], k in [0, taps-1): the input at position ctx - (taps-1) + k (zero before the start)
+template <typename TO>
+__global__ void canon_conv_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ state,
+                                  const int32_t* __restrict__ qsl, const int32_t* __restrict__ seq_lens,
+                                  const int32_t* __restrict__ slots, TO* __restrict__ out, int W, int taps, int tile,
+                                  int write_state) {
+  const int s = blockIdx.z;
+  const int q0 = qsl[s], q = qsl[s + 1] - q0, slot = slots[s];
+  if (slot < 0 || q <= 0) return;
+  const int t0 = blockIdx.y * tile;
+  if (t0 >= q) return;
+  const int t1 = min(q, t0 + tile);
+  const int ctx = seq_lens[s] - q;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= W) return;
+  const int nh = taps - 1;
+  float hist[kMaxTaps - 1], wt[kMaxTaps];
+#pragma unroll
+  for (int j = 0; j < kMaxTaps; ++j) wt[j] = j < taps ? w[(int64_t)c * taps + j] : 0.f;
+  float* st = state + ((int64_t)slot * nh) * W + c;
+#pragma unroll
+  for (int j = 0; j < kMaxTaps - 1; ++j) {
+    float v = 0.f;
+    if (j < nh) {
+      const int li = t0 - nh + j;  // local index of the input this tap history starts with
+      if (li >= 0) v = x[(int64_t)(q0 + li) * W + c];
+      else if (ctx + li >= 0) v = st[(int64_t)(nh + li) * W];
+    }
+    hist[j] = v;
+  }
+  for (int t = t0; t < t1; ++t) {
+    const float cur = x[(int64_t)(q0 + t) * W + c];
+    float acc = cur;
+#pragma unroll
+    for (int j = 0; j < kMaxTaps - 1; ++j)
+      if (j < nh) acc += wt[j] * hist[j];
+    acc += wt[nh] * cur;
+    stf(out + (int64_t)(q0 + t) * W + c, acc);
+#pragma unroll
+    for (int j = 0; j < kMaxTaps - 1; ++j) {  // shift; the newest input goes last
+      const float nxt = j + 1 < kMaxTaps - 1 ? hist[j + 1] : 0.f;
+      hist[j] = j == nh - 1 ? cur : nxt;
+    }
+  }
+  if (write_state) {
+#pragma unroll
+    for (int j = 0; j < kMaxTaps - 1; ++j)
+      if (j < nh) st[(int64_t)j * W] = hist[j];
+  }
+}
+
+// the carried rows after a step whose sequences were convolved by several tiles
+__global__ void canon_state_kernel(const float* __restrict__ x, float* __restrict__ state, const int32_t* __restrict__ qsl,
+                                   const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots, int W,
+                                   int taps) {
+  const int s = blockIdx.y;
+  const int q0 = qsl[s], q = qsl[s + 1] - q0, slot = slots[s];
+  if (slot < 0 || q <= 0) return;
+  const int ctx = seq_lens[s] - q;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= W) return;
+  const int nh = taps - 1;
+  float* st = state + ((int64_t)slot * nh) * W + c;
+  float v[kMaxTaps - 1];
+#pragma unroll
+  for (int j = 0; j < kMaxTaps - 1; ++j) {
+    v[j] = 0.f;
+    if (j < nh) {
+      const int li = q - nh + j;
+      if (li >= 0) v[j] = x[(int64_t)(q0 + li) * W + c];
+      else if (ctx + li >= 0) v[j] = st[(int64_t)(nh + li) * W];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kMaxTaps - 1; ++j)
+    if (j < nh) st[(int64_t)j * W] = v[j];
+}
+
+// ------------------------------------------------------------------ norm after the (scaled) residual sum
+template <typename TY, typename TO>
+__global__ __launch_bounds__(256) void scaled_add_rmsnorm_kernel(const float* x, const TY* __restrict__ y,
+                                                                 int64_t y_stride, const float* __restrict__ bias,
+                                                                 float alpha, const float* __restrict__ w, float w_offset,
+                                                                 float eps, float* x_out,
+                                                                 TO* __restrict__ out, int W) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const float* xr = x + (int64_t)t * W;
+  const TY* yr = y ? y + (int64_t)t * y_stride : nullptr;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = alpha * xr[c];
+    if (yr) v += ldf(yr + c);
+    if (bias) v += bias[c];
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = alpha * xr[c];
+    if (yr) v += ldf(yr + c);
+    if (bias) v += bias[c];
+    const float o = v * r * (w_offset + w[c]);
+    if (x_out) x_out[(int64_t)t * W + c] = o;
+    if (out) stf(out + (int64_t)t * W + c, o);
+  }
+}
+
+// ------------------------------------------------------------------ latent attention: projections -> cache
+// proj row: [.. | q latent (Rq) at off_q | kv latent (R) + shared rotary key (rd) at off_kv | ..]
+// rot table: [positions][rot_dims/2][2] = (cos, sin) of position * base^(-2i/rot_dims)
+template <typename T>
+__global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ proj, int64_t ld, int off_q, int Rq,
+                                                          int off_kv, int R, int rd, const float* __restrict__ wq,
+                                                          const float* __restrict__ wkv, float eps,
+                                                          const int32_t* __restrict__ positions,
+                                                          const int32_t* __restrict__ slot_mapping,
+                                                          const float* __restrict__ rot, int rot_dims,
+                                                          T* __restrict__ cq, T* __restrict__ cache) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const T* row = proj + (int64_t)t * ld;
+  {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < Rq; i += blockDim.x) {
+      const float v = ldf(row + off_q + i);
+      ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float r = 1.f / sqrtf(ss / (float)Rq + eps);
+    for (int i = threadIdx.x; i < Rq; i += blockDim.x) stf(cq + (int64_t)t * Rq + i, ldf(row + off_q + i) * r * wq[i]);
+  }
+  if (off_kv < 0) return;
+  const int slot = slot_mapping[t];
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < R; i += blockDim.x) {
+    const float v = ldf(row + off_kv + i);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  if (slot < 0) return;
+  const float r = 1.f / sqrtf(ss / (float)R + eps);
+  T* dst = cache + (int64_t)slot * (R + rd);
+  for (int i = threadIdx.x; i < R; i += blockDim.x) stf(dst + i, ldf(row + off_kv + i) * r * wkv[i]);
+  const int pos = positions[t];
+  const int half = rot_dims >> 1;
+  const T* kr = row + off_kv + R;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float c = rot[((int64_t)pos * half + i) * 2], s = rot[((int64_t)pos * half + i) * 2 + 1];
+    const float u = ldf(kr + 2 * i), v = ldf(kr + 2 * i + 1);
+    stf(dst + R + 2 * i, u * c - v * s);
+    stf(dst + R + 2 * i + 1, v * c + u * s);
+  }
+  for (int i = rot_dims + threadIdx.x; i < rd; i += blockDim.x) stf(dst + R + i, ldf(kr + i));
+}
+
+// ------------------------------------------------------------------ latent attention over the paged latent cache
+// Every head scores the same cached row [kv latent (R) | rotated key (rd)]: the query is
+// [W_uk^T q_unrotated (R) | rotated q (rd)], the value is the latent itself, and the
+// per-head value projection follows as a GEMM. One workgroup = one token x kHPB heads;
+// a tile of KT keys is staged in LDS once and read by all its heads.
+constexpr int kHPB = 8;  // heads per workgroup (4 waves x 2)
+
+template <typename T, int NR>
+__global__ __launch_bounds__(256) void latent_attention_kernel(
+    const T* __restrict__ qabs, const T* __restrict__ q, int64_t q_stride, int dq, int dn, const T* __restrict__ gate,
+    int64_t gate_stride, const T* __restrict__ cache, const int32_t* __restrict__ block_tables, int bt_width, int bs,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ token_seq, const float* __restrict__ rot,
+    int rot_dims, T* __restrict__ out, int Ttot, int H, int R, int rd, int window, float scale, int KT) {
+  extern __shared__ float smem[];
+  const int Dk = R + rd, ldt = Dk + 1;
+  float* tile = smem;                      // [KT][Dk + 1]
+  float* qs = smem + (size_t)KT * ldt;     // [kHPB][Dk]
+  const int t = blockIdx.x, hb = blockIdx.y * kHPB;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int s = token_seq[t];
+  if (s < 0) {
+    for (int hl = wave; hl < kHPB && hb + hl < H; hl += 4)
+      for (int d = lane; d < R; d += 64) stf(out + ((int64_t)(hb + hl) * Ttot + t) * R + d, 0.f);
+    return;
+  }
+  const int pos = positions[t];
+  const int j0 = max(0, pos - window + 1);
+  // queries of this workgroup's heads -> LDS (scaled; rotated part rotated here)
+  const int half = rot_dims >> 1;
+  for (int hl = wave; hl < kHPB; hl += 4) {
+    const int h = hb + hl;
+    float* qh = qs + hl * Dk;
+    if (h >= H) {
+      for (int d = lane; d < Dk; d += 64) qh[d] = 0.f;
+      continue;
+    }
+    for (int d = lane; d < R; d += 64) qh[d] = ldf(qabs + ((int64_t)h * Ttot + t) * R + d) * scale;
+    const T* qr = q + (int64_t)t * q_stride + (int64_t)h * dq + dn;
+    for (int i = lane; i < half; i += 64) {
+      const float c = rot[((int64_t)pos * half + i) * 2], sn = rot[((int64_t)pos * half + i) * 2 + 1];
+      const float u = ldf(qr + 2 * i), v = ldf(qr + 2 * i + 1);
+      qh[R + 2 * i] = (u * c - v * sn) * scale;
+      qh[R + 2 * i + 1] = (v * c + u * sn) * scale;
+    }
+    for (int i = rot_dims + lane; i < rd; i += 64) qh[R + i] = ldf(qr + i) * scale;
+  }
+  const int LPK = 64 / KT;  // lanes per key in the score phase
+  const int kj = lane / LPK, part = lane % LPK;
+  float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+  float acc[2][NR];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int i = 0; i < NR; ++i) acc[a][i] = 0.f;
+  const int32_t* bt = block_tables + (int64_t)s * bt_width;
+  for (int k0 = j0; k0 <= pos; k0 += KT) {
+    const int n = min(KT, pos - k0 + 1);
+    __syncthreads();  // the previous tile is consumed (and qs is written, first time round)
+    for (int jj = wave; jj < n; jj += 4) {
+      const int key = k0 + jj;
+      const T* src = cache + ((int64_t)bt[key / bs] * bs + key % bs) * Dk;
+      for (int d = lane; d < Dk; d += 64) tile[jj * ldt + d] = ldf(src + d);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      const int hl = wave + 4 * a;
+      if (hb + hl >= H) continue;
+      const float* qh = qs + hl * Dk;
+      float sc = 0.f;
+      if (kj < n) {
+        const float* kr = tile + kj * ldt;
+        for (int d = part; d < Dk; d += LPK) sc += qh[d] * kr[d];
+      }
+      for (int o = 1; o < LPK; o <<= 1) sc += __shfl_xor(sc, o, 64);
+      if (kj >= n) sc = -INFINITY;
+      const float mn = fmaxf(m[a], wave_max(sc));
+      const float p = kj < n ? expf(sc - mn) : 0.f;
+      const float corr = m[a] == -INFINITY ? 0.f : expf(m[a] - mn);
+      l[a] = l[a] * corr + wave_sum(part == 0 ? p : 0.f);
+      m[a] = mn;
+#pragma unroll
+      for (int i = 0; i < NR; ++i) acc[a][i] *= corr;
+      for (int j = 0; j < n; ++j) {
+        const float pj = __shfl(p, j * LPK, 64);
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+          const int d = lane + 64 * i;
+          if (d < R) acc[a][i] += pj * tile[j * ldt + d];
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    const int h = hb + wave + 4 * a;
+    if (h >= H) continue;
+    const float g = sigmoidf(ldf(gate + (int64_t)t * gate_stride + h)) / l[a];
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int d = lane + 64 * i;
+      if (d < R) stf(out + ((int64_t)h * Ttot + t) * R + d, acc[a][i] * g);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ generalized delta rule
+// One workgroup = (head, sequence); thread (col, ks) owns rows ks, ks + 4, .. of column col
+// of the [D x D] state, so u^T S and S^T r reduce over 4 neighbouring lanes only.
+constexpr int kKS = 4;
+
+template <typename T, int MAXR>
+__global__ void delta_scan_kernel(const T* __restrict__ proj, int64_t ld, int off_r, int off_k, int off_v, int off_a,
+                                  const T* __restrict__ wl, int64_t ld_wl, const float* __restrict__ a_bias,
+                                  const float* __restrict__ w0, float* __restrict__ state,
+                                  const int32_t* __restrict__ qsl, const int32_t* __restrict__ seq_lens,
+                                  const int32_t* __restrict__ slots, float* __restrict__ o, int H, int D) {
+  const int h = blockIdx.x, s = blockIdx.y;
+  const int q0 = qsl[s], q = qsl[s + 1] - q0, slot = slots[s];
+  if (slot < 0 || q <= 0) return;
+  const int ctx = seq_lens[s] - q;
+  const int col = threadIdx.x / kKS, ks = threadIdx.x % kKS;
+  const bool live = col < D;
+  const int cc = live ? col : 0;
+  float S[MAXR], ab[MAXR], wb[MAXR];
+  float* st = state + ((int64_t)slot * H + h) * D * D;
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    const int i = ks + kKS * r;
+    const bool ok = i < D;
+    S[r] = (ok && ctx > 0) ? st[(int64_t)i * D + cc] : 0.f;
+    ab[r] = ok ? a_bias[h * D + i] : 0.f;
+    wb[r] = ok ? w0[h * D + i] : 0.f;
+  }
+  const int HD = H * D;
+  for (int t = 0; t < q; ++t) {
+    const T* row = proj + (int64_t)(q0 + t) * ld + h * D;
+    const T* wrow = wl + (int64_t)(q0 + t) * ld_wl + h * D;
+    float kk[MAXR], ksq = 0.f;
+#pragma unroll
+    for (int r = 0; r < MAXR; ++r) {
+      const int i = ks + kKS * r;
+      kk[r] = i < D ? ldf(row + off_k + i) : 0.f;
+      ksq += kk[r] * kk[r];
+    }
+    ksq += __shfl_xor(ksq, 1, 64);
+    ksq += __shfl_xor(ksq, 2, 64);
+    const float inv = 1.f / sqrtf(ksq + 1e-6f);
+    float uS = 0.f;
+#pragma unroll
+    for (int r = 0; r < MAXR; ++r) uS += kk[r] * inv * S[r];
+    uS += __shfl_xor(uS, 1, 64);
+    uS += __shfl_xor(uS, 2, 64);
+    const float v = ldf(row + off_v + cc);
+    float ot = 0.f;
+#pragma unroll
+    for (int r = 0; r < MAXR; ++r) {
+      const int i = ks + kKS * r;
+      if (i < D) {
+        const float u = kk[r] * inv;
+        const float w = expf(-0.6065306597126334f * sigmoidf(ldf(wrow + i) + wb[r]));
+        const float a = sigmoidf(ldf(row + off_a + i) + ab[r]);
+        S[r] = w * S[r] - a * u * uS + kk[r] * v;
+        ot += S[r] * ldf(row + off_r + i);
+      }
+    }
+    ot += __shfl_xor(ot, 1, 64);
+    ot += __shfl_xor(ot, 2, 64);
+    if (live && ks == 0) o[(int64_t)(q0 + t) * HD + h * D + col] = ot;
+  }
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < MAXR; ++r) {
+      const int i = ks + kKS * r;
+      if (i < D) st[(int64_t)i * D + col] = S[r];
+    }
+  }
+}
+
+template <typename T>
+__global__ void delta_out_kernel(const float* __restrict__ o, const float* __restrict__ nw, const T* __restrict__ gate,
+                                 int64_t gate_stride, float eps, T* __restrict__ out, int H, int D) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* row = o + ((int64_t)t * H + h) * D;
+  float ss = 0.f;
+  for (int d = lane; d < D; d += 64) ss += row[d] * row[d];
+  ss = wave_sum(ss);
+  const float r = 1.f / sqrtf(ss / (float)D + eps);
+  for (int d = lane; d < D; d += 64)
+    stf(out + ((int64_t)t * H + h) * D + d,
+        row[d] * r * nw[h * D + d] * sigmoidf(ldf(gate + (int64_t)t * gate_stride + h * D + d)));
+}
+
+// ------------------------------------------------------------------ activations
+// xIELU with sp = softplus(p), cn = 1/2 + softplus(q):
+//   z > 0: sp z^2 + z/2 ;  z <= 0: cn (exp(z) - 1 - z) + z/2
+template <typename T>
+__global__ void xielu_kernel(const T* __restrict__ in, const float* __restrict__ bias, float sp, float cn,
+                             T* __restrict__ out, int64_t n, int F) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    float z = ldf(in + i);
+    if (bias) z += bias[i % F];
+    const float y = z > 0.f ? sp * z * z + 0.5f * z : cn * (expm1f(z) - z) + 0.5f * z;
+    stf(out + i, y);
+  }
+}
+
+template <typename T>
+__global__ void tanh_cols_kernel(const T* __restrict__ in, int64_t ld, T* __restrict__ out, int n, int64_t total) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x)
+    stf(out + i, tanhf(ldf(in + (i / n) * ld + i % n)));
+}
+
+// [H, T, n] -> [T, H * n]
+template <typename T>
+__global__ void heads_to_rows_kernel(const T* __restrict__ in, T* __restrict__ out, int Ttot, int H, int n) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < H * n; i += blockDim.x) {
+    const int h = i / n, d = i % n;
+    out[(int64_t)t * H * n + i] = in[((int64_t)h * Ttot + t) * n + d];
+  }
+}
+
+// ================================================================== host launchers
+#define XGM_DISPATCH_T(f32, ...)      \
+  if (f32) {                          \
+    using T = float;                  \
+    __VA_ARGS__                       \
+  } else {                            \
+    using T = bf16;                   \
+    __VA_ARGS__                       \
+  }
+
+void embed_rows(const int32_t* ids, const void* table, bool f32, float* out, int T_, int W, int V, hipStream_t st) {
+  if (T_ <= 0) return;
+  XGM_DISPATCH_T(f32, embed_rows_kernel<T><<<T_, 256, 0, st>>>(ids, (const T*)table, out, W, V);)
+}
+
+void canon_conv(const float* x, const float* w, float* state, const int32_t* qsl, const int32_t* seq_lens,
+                const int32_t* slots, void* out, bool out_f32, int ns, int max_q, int W, int taps, hipStream_t st) {
+  if (ns <= 0 || max_q <= 0) return;
+  const int tile = 64;
+  const int ntiles = (max_q + tile - 1) / tile;
+  dim3 grid((W + 255) / 256, ntiles, ns);
+  const int ws = ntiles == 1 ? 1 : 0;
+  XGM_DISPATCH_T(out_f32, canon_conv_kernel<T><<<grid, 256, 0, st>>>(x, w, state, qsl, seq_lens, slots, (T*)out, W, taps,
+                                                                      tile, ws);)
+  if (!ws) canon_state_kernel<<<dim3((W + 255) / 256, ns), 256, 0, st>>>(x, state, qsl, seq_lens, slots, W, taps);
+}
+
+void scaled_add_rmsnorm(const float* x, const void* y, bool y_f32, int64_t y_stride, const float* bias, float alpha,
+                        const float* w, float w_offset, float eps, float* x_out, void* out, bool out_f32, int T_, int W,
+                        hipStream_t st) {
+  if (T_ <= 0) return;
+#define XGM_SAR(TY, TO) \
+  scaled_add_rmsnorm_kernel<TY, TO><<<T_, 256, 0, st>>>(x, (const TY*)y, y_stride, bias, alpha, w, w_offset, eps, x_out, (TO*)out, W)
+  if (y_f32) {
+    if (out_f32) XGM_SAR(float, float); else XGM_SAR(float, bf16);
+  } else {
+    if (out_f32) XGM_SAR(bf16, float); else XGM_SAR(bf16, bf16);
+  }
+#undef XGM_SAR
+}
+
+void latent_prep(const void* proj, bool f32, int64_t ld, int off_q, int Rq, int off_kv, int R, int rd, const float* wq,
+                 const float* wkv, float eps, const int32_t* positions, const int32_t* slot_mapping, const float* rot,
+                 int rot_dims, void* cq, void* cache, int T_, hipStream_t st) {
+  if (T_ <= 0) return;
+  XGM_DISPATCH_T(f32, latent_prep_kernel<T><<<T_, 256, 0, st>>>((const T*)proj, ld, off_q, Rq, off_kv, R, rd, wq, wkv, eps,
+                                                                 positions, slot_mapping, rot, rot_dims, (T*)cq,
+                                                                 (T*)cache);)
+}
+
+template <typename T, int NR>
+static int launch_latent_attention(const void* qabs, const void* q, int64_t q_stride, int dq, int dn, const void* gate,
+                                   int64_t gate_stride, const void* cache, const int32_t* bt, int bt_width, int bs,
+                                   const int32_t* positions, const int32_t* token_seq, const float* rot, int rot_dims,
+                                   void* out, int Ttot, int H, int R, int rd, int window, float scale, hipStream_t st) {
+  const int Dk = R + rd;
+  int KT = 64;
+  auto bytes = [&](int kt) { return ((size_t)kt * (Dk + 1) + (size_t)kHPB * Dk) * sizeof(float); };
+  while (KT > 16 && bytes(KT) > 96 * 1024) KT >>= 1;
+  if (bytes(KT) > 150 * 1024) return -1;
+  while (KT > 16 && KT / 2 >= window) KT >>= 1;  // short windows: no idle key lanes
+  auto kern = latent_attention_kernel<T, NR>;
+  if (bytes(KT) > 48 * 1024) {
+    static size_t set_bytes = 0;
+    if (bytes(KT) > set_bytes) {
+      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
+        return -2;
+      set_bytes = 150 * 1024;
+    }
+  }
+  dim3 grid(Ttot, (H + kHPB - 1) / kHPB);
+  kern<<<grid, 256, bytes(KT), st>>>((const T*)qabs, (const T*)q, q_stride, dq, dn, (const T*)gate, gate_stride,
+                                     (const T*)cache, bt, bt_width, bs, positions, token_seq, rot, rot_dims, (T*)out, Ttot,
+                                     H, R, rd, window, scale, KT);
+  return 0;
+}
+
+int latent_attention(const void* qabs, const void* q, bool f32, int64_t q_stride, int dq, int dn, const void* gate,
+                     int64_t gate_stride, const void* cache, const int32_t* bt, int bt_width, int bs,
+                     const int32_t* positions, const int32_t* token_seq, const float* rot, int rot_dims, void* out,
+                     int Ttot, int H, int R, int rd, int window, float scale, hipStream_t st) {
+  if (Ttot <= 0) return 0;
+#define XGM_LA(NR)                                                                                                  \
+  XGM_DISPATCH_T(f32, return (launch_latent_attention<T, NR>(qabs, q, q_stride, dq, dn, gate, gate_stride, cache, bt, \
+                                                              bt_width, bs, positions, token_seq, rot, rot_dims, out, \
+                                                              Ttot, H, R, rd, window, scale, st));)
+  if (R <= 128) { XGM_LA(2) }
+  if (R <= 256) { XGM_LA(4) }
+  if (R <= 512) { XGM_LA(8) }
+  if (R <= 1024) { XGM_LA(16) }
+#undef XGM_LA
+  return -3;
+}
+
+int delta_scan(const void* proj, bool f32, int64_t ld, int off_r, int off_k, int off_v, int off_a, const void* wl,
+               int64_t ld_wl, const float* a_bias, const float* w0, float* state, const int32_t* qsl,
+               const int32_t* seq_lens, const int32_t* slots, float* o, int ns, int H, int D, hipStream_t st) {
+  if (ns <= 0) return 0;
+  const int threads = ((kKS * D + 63) / 64) * 64;
+  if (threads > 1024) return -1;
+  dim3 grid(H, ns);
+#define XGM_DS(MAXR)                                                                                                  \
+  XGM_DISPATCH_T(f32, delta_scan_kernel<T, MAXR><<<grid, threads, 0, st>>>((const T*)proj, ld, off_r, off_k, off_v,  \
+                                                                            off_a, (const T*)wl, ld_wl, a_bias, w0,   \
+                                                                            state, qsl, seq_lens, slots, o, H, D);)  \
+  return 0;
+  if (D <= 32) { XGM_DS(8) }
+  if (D <= 64) { XGM_DS(16) }
+  if (D <= 128) { XGM_DS(32) }
+  if (D <= 256) { XGM_DS(64) }
+#undef XGM_DS
+  return -1;
+}
+
+void delta_out(const float* o, const float* nw, const void* gate, bool f32, int64_t gate_stride, float eps, void* out,
+               int T_, int H, int D, hipStream_t st) {
+  if (T_ <= 0) return;
+  XGM_DISPATCH_T(f32, delta_out_kernel<T><<<dim3(T_, H), 64, 0, st>>>(o, nw, (const T*)gate, gate_stride, eps, (T*)out, H, D);)
+}
+
+void xielu(const void* in, bool f32, const float* bias, float sp, float cn, void* out, int64_t n, int F, hipStream_t st) {
+  if (n <= 0) return;
+  const int blocks = (int)std::min<int64_t>((n + 255) / 256, 65535);
+  XGM_DISPATCH_T(f32, xielu_kernel<T><<<blocks, 256, 0, st>>>((const T*)in, bias, sp, cn, (T*)out, n, F);)
+}
+
+void tanh_cols(const void* in, bool f32, int64_t ld, void* out, int T_, int n, hipStream_t st) {
+  const int64_t total = (int64_t)T_ * n;
+  if (total <= 0) return;
+  const int blocks = (int)std::min<int64_t>((total + 255) / 256, 65535);
+  XGM_DISPATCH_T(f32, tanh_cols_kernel<T><<<blocks, 256, 0, st>>>((const T*)in, ld, (T*)out, n, total);)
+}
+
+void heads_to_rows(const void* in, bool f32, void* out, int T_, int H, int n, hipStream_t st) {
+  if (T_ <= 0) return;
+  XGM_DISPATCH_T(f32, heads_to_rows_kernel<T><<<T_, 256, 0, st>>>((const T*)in, (T*)out, T_, H, n);)
+}
+
+}  // namespace xgm

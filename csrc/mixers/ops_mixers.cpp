@@ -1,0 +1,107 @@
+// pybind11 entry points of xgserve._mixers: raw device pointers + the caller's hipStream_t
+// (graph-capturable, no dependence on torch's C++ ABI). Shapes are checked here, before launch.
+#include <hip/hip_runtime.h>
+#include <pybind11/pybind11.h>
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+namespace py = pybind11;
+
+namespace xgm {
+void embed_rows(const int32_t*, const void*, bool, float*, int, int, int, hipStream_t);
+void canon_conv(const float*, const float*, float*, const int32_t*, const int32_t*, const int32_t*, void*, bool, int, int,
+                int, int, hipStream_t);
+void scaled_add_rmsnorm(const float*, const void*, bool, int64_t, const float*, float, const float*, float, float, float*,
+                        void*, bool, int, int, hipStream_t);
+void latent_prep(const void*, bool, int64_t, int, int, int, int, int, const float*, const float*, float, const int32_t*,
+                 const int32_t*, const float*, int, void*, void*, int, hipStream_t);
+int latent_attention(const void*, const void*, bool, int64_t, int, int, const void*, int64_t, const void*, const int32_t*,
+                     int, int, const int32_t*, const int32_t*, const float*, int, void*, int, int, int, int, int, float,
+                     hipStream_t);
+int delta_scan(const void*, bool, int64_t, int, int, int, int, const void*, int64_t, const float*, const float*, float*,
+               const int32_t*, const int32_t*, const int32_t*, float*, int, int, int, hipStream_t);
+void delta_out(const float*, const float*, const void*, bool, int64_t, float, void*, int, int, int, hipStream_t);
+void xielu(const void*, bool, const float*, float, float, void*, int64_t, int, hipStream_t);
+void tanh_cols(const void*, bool, int64_t, void*, int, int, hipStream_t);
+void heads_to_rows(const void*, bool, void*, int, int, int, hipStream_t);
+}  // namespace xgm
+
+template <typename T> static T* P(uintptr_t p) { return reinterpret_cast<T*>(p); }
+static hipStream_t S(uintptr_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+static void check(int rc, const char* what) {
+  if (rc != 0) throw std::invalid_argument(std::string(what) + ": unsupported shape (code " + std::to_string(rc) + ")");
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+PYBIND11_MODULE(_mixers, m) {
+  m.def("embed_rows", [](uintptr_t ids, uintptr_t table, bool f32, uintptr_t out, int T, int W, int V, uintptr_t st) {
+    xgm::embed_rows(P<const int32_t>(ids), P<const void>(table), f32, P<float>(out), T, W, V, S(st));
+    check(0, "embed_rows");
+  });
+  m.def("canon_conv", [](uintptr_t x, uintptr_t w, uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots,
+                         uintptr_t out, bool out_f32, int ns, int max_q, int W, int taps, uintptr_t st) {
+    if (taps < 1 || taps > 8) throw std::invalid_argument("canon_conv: taps must be in [1, 8]");
+    xgm::canon_conv(P<const float>(x), P<const float>(w), P<float>(state), P<const int32_t>(qsl), P<const int32_t>(sl),
+                    P<const int32_t>(slots), P<void>(out), out_f32, ns, max_q, W, taps, S(st));
+    check(0, "canon_conv");
+  });
+  m.def("scaled_add_rmsnorm", [](uintptr_t x, uintptr_t y, bool y_f32, int64_t y_stride, uintptr_t bias, float alpha,
+                                 uintptr_t w, float w_offset, float eps, uintptr_t x_out, uintptr_t out, bool out_f32,
+                                 int T, int W, uintptr_t st) {
+    xgm::scaled_add_rmsnorm(P<const float>(x), P<const void>(y), y_f32, y_stride, P<const float>(bias), alpha,
+                            P<const float>(w), w_offset, eps, P<float>(x_out), P<void>(out), out_f32, T, W, S(st));
+    check(0, "scaled_add_rmsnorm");
+  });
+  m.def("latent_prep", [](uintptr_t proj, bool f32, int64_t ld, int off_q, int Rq, int off_kv, int R, int rd, uintptr_t wq,
+                          uintptr_t wkv, float eps, uintptr_t pos, uintptr_t slot_mapping, uintptr_t rot, int rot_dims,
+                          uintptr_t cq, uintptr_t cache, int T, uintptr_t st) {
+    if (rot_dims % 2 || rot_dims > rd) throw std::invalid_argument("latent_prep: rot_dims must be even and <= rd");
+    xgm::latent_prep(P<const void>(proj), f32, ld, off_q, Rq, off_kv, R, rd, P<const float>(wq), P<const float>(wkv), eps,
+                     P<const int32_t>(pos), P<const int32_t>(slot_mapping), P<const float>(rot), rot_dims, P<void>(cq),
+                     P<void>(cache), T, S(st));
+    check(0, "latent_prep");
+  });
+  m.def("latent_attention", [](uintptr_t qabs, uintptr_t q, bool f32, int64_t q_stride, int dq, int dn, uintptr_t gate,
+                               int64_t gate_stride, uintptr_t cache, uintptr_t bt, int bt_width, int bs, uintptr_t pos,
+                               uintptr_t token_seq, uintptr_t rot, int rot_dims, uintptr_t out, int T, int H, int R, int rd,
+                               int window, float scale, uintptr_t st) {
+    if (rot_dims % 2 || rot_dims > rd || dn + rd != dq || window < 1 || bs < 1)
+      throw std::invalid_argument("latent_attention: inconsistent sizes");
+    int rc = xgm::latent_attention(P<const void>(qabs), P<const void>(q), f32, q_stride, dq, dn, P<const void>(gate),
+                                   gate_stride, P<const void>(cache), P<const int32_t>(bt), bt_width, bs,
+                                   P<const int32_t>(pos), P<const int32_t>(token_seq), P<const float>(rot), rot_dims,
+                                   P<void>(out), T, H, R, rd, window, scale, S(st));
+    check(rc, "latent_attention");
+  });
+  m.def("delta_scan", [](uintptr_t proj, bool f32, int64_t ld, int off_r, int off_k, int off_v, int off_a, uintptr_t wl,
+                         int64_t ld_wl, uintptr_t a_bias, uintptr_t w0, uintptr_t state, uintptr_t qsl, uintptr_t sl,
+                         uintptr_t slots, uintptr_t o, int ns, int H, int D, uintptr_t st) {
+    int rc = xgm::delta_scan(P<const void>(proj), f32, ld, off_r, off_k, off_v, off_a, P<const void>(wl), ld_wl,
+                             P<const float>(a_bias), P<const float>(w0), P<float>(state), P<const int32_t>(qsl),
+                             P<const int32_t>(sl), P<const int32_t>(slots), P<float>(o), ns, H, D, S(st));
+    check(rc, "delta_scan");
+  });
+  m.def("delta_out", [](uintptr_t o, uintptr_t nw, uintptr_t gate, bool f32, int64_t gate_stride, float eps, uintptr_t out,
+                        int T, int H, int D, uintptr_t st) {
+    xgm::delta_out(P<const float>(o), P<const float>(nw), P<const void>(gate), f32, gate_stride, eps, P<void>(out), T, H, D,
+                   S(st));
+    check(0, "delta_out");
+  });
+  m.def("xielu", [](uintptr_t in, bool f32, uintptr_t bias, float sp, float cn, uintptr_t out, int64_t n, int F,
+                    uintptr_t st) {
+    xgm::xielu(P<const void>(in), f32, P<const float>(bias), sp, cn, P<void>(out), n, F, S(st));
+    check(0, "xielu");
+  });
+  m.def("tanh_cols", [](uintptr_t in, bool f32, int64_t ld, uintptr_t out, int T, int n, uintptr_t st) {
+    xgm::tanh_cols(P<const void>(in), f32, ld, P<void>(out), T, n, S(st));
+    check(0, "tanh_cols");
+  });
+  m.def("heads_to_rows", [](uintptr_t in, bool f32, uintptr_t out, int T, int H, int n, uintptr_t st) {
+    xgm::heads_to_rows(P<const void>(in), f32, P<void>(out), T, H, n, S(st));
+    check(0, "heads_to_rows");
+  });
+}

@@ -257,6 +257,11 @@ PYBIND11_MODULE(_runtime, m) {
                                          f.num_cached));
              return out;
            })
+      .def("extend", &StepScheduler::extend)
+      .def("schedule_rows",
+           [](StepScheduler& s, const std::vector<int64_t>& ids, const std::vector<int32_t>& counts,
+              const std::vector<std::vector<int32_t>>& want) { return plan_dict(s.schedule_rows(ids, counts, want)); })
+      .def("advance", &StepScheduler::advance)
       .def("lookahead", &StepScheduler::lookahead, py::arg("across_length_finish") = false)
       .def("commit",
            [](StepScheduler& s, py::array_t<int32_t, py::array::c_style | py::array::forcecast> tok) {

@@ -352,6 +352,77 @@ const StepPlan& StepScheduler::schedule() {
   return plan_;
 }
 
+void StepScheduler::extend(int64_t id, const std::vector<int32_t>& tokens) {
+  auto it = seqs_.find(id);
+  if (it == seqs_.end()) {
+    if (static_cast<int>(running_.size()) >= cfg_.max_num_seqs || free_slots_.empty())
+      throw std::runtime_error("replay: no free sequence slot");
+    auto s = std::make_unique<Sequence>();
+    s->id = id;
+    s->arrival = arrival_counter_++;
+    s->ignore_eos = true;
+    s->max_tokens = 0;
+    s->status = SeqStatus::Running;
+    s->slot = free_slots_.back();
+    free_slots_.pop_back();
+    running_.push_back(s.get());
+    it = seqs_.emplace(id, std::move(s)).first;
+  }
+  Sequence& s = *it->second;
+  if (static_cast<int>(s.tokens.size() + tokens.size()) > cfg_.max_model_len)
+    throw std::runtime_error("replay: sequence exceeds max_model_len");
+  s.tokens.insert(s.tokens.end(), tokens.begin(), tokens.end());
+  s.prompt_len = static_cast<int>(s.tokens.size());
+}
+
+const StepPlan& StepScheduler::schedule_rows(const std::vector<int64_t>& ids, const std::vector<int32_t>& counts,
+                                             const std::vector<std::vector<int32_t>>& want) {
+  if (ids.size() != counts.size() || ids.size() != want.size())
+    throw std::invalid_argument("replay: ids / counts / want differ in length");
+  plan_ = StepPlan{};
+  plan_.query_start_loc.push_back(0);
+  plan_seqs_.clear();
+  for (int pass = 0; pass < 2; ++pass) {  // single tokens behind a context first
+    for (size_t i = 0; i < ids.size(); ++i) {
+      auto it = seqs_.find(ids[i]);
+      if (it == seqs_.end()) throw std::invalid_argument("replay: unknown sequence");
+      Sequence& s = *it->second;
+      const int q = counts[i];
+      const bool decode = q == 1 && s.num_computed > 0;
+      if (decode != (pass == 0)) continue;
+      if (q < 1 || s.num_computed + q > static_cast<int>(s.tokens.size()))
+        throw std::invalid_argument("replay: a row asks for tokens the sequence does not have");
+      for (const Sequence* other : plan_seqs_)
+        if (other == &s) throw std::invalid_argument("replay: a sequence appears twice in a step");
+      if (!ensure_blocks(s, s.num_computed + q)) throw std::runtime_error("replay: out of cache pages");
+      const int base = plan_.num_tokens;
+      emit(s, q, !decode, false);
+      for (int32_t w : want[i]) {
+        if (w < 0 || w >= q) throw std::invalid_argument("replay: a wanted row lies outside its tokens");
+        plan_.logits_indices.push_back(base + w);
+      }
+    }
+    if (pass == 0) plan_.num_decodes = plan_.num_seqs;
+  }
+  int w = 1;
+  for (Sequence* s : plan_seqs_) w = std::max<int>(w, static_cast<int>(s->blocks.size()));
+  plan_.bt_width = w;
+  plan_.block_tables.assign(static_cast<size_t>(plan_.num_seqs) * w, 0);
+  for (int i = 0; i < plan_.num_seqs; ++i) {
+    const auto& b = plan_seqs_[i]->blocks;
+    std::copy(b.begin(), b.end(), plan_.block_tables.begin() + static_cast<size_t>(i) * w);
+  }
+  return plan_;
+}
+
+void StepScheduler::advance() {
+  for (int i = 0; i < plan_.num_seqs; ++i) {
+    Sequence* s = plan_seqs_[i];
+    if (s != nullptr && s->status == SeqStatus::Running) s->num_computed += plan_.q_lens[i];
+  }
+  for (auto& q : plan_seqs_) q = nullptr;
+}
+
 int StepScheduler::check_stop(Sequence& s) {
   const int32_t last = s.tokens.back();
   const int gen = s.num_generated();

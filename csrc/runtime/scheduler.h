@@ -155,6 +155,19 @@ class StepScheduler {
   std::vector<FinishedSeq> commit(const int32_t* tokens, int num_sample);
   int num_inflight() const { return static_cast<int>(inflight_.size()); }
 
+  // Replay (teacher-forced) scheduling: the caller dictates every step's rows, e.g. to
+  // replay a recorded trace or to score given text. extend() appends known tokens to a
+  // sequence (creating it on first use; it takes a state slot and pages like any admitted
+  // sequence); schedule_rows() plans exactly `counts[i]` next tokens of `ids[i]` -- rows of
+  // one token behind a non-empty context first, as in every plan -- with the step's logits
+  // rows at `want[i]` (offsets into the row's tokens); advance() marks the planned tokens
+  // computed. Nothing is sampled, preempted or evicted: running out of pages or slots throws.
+  // abort() ends a sequence and returns its slot and pages.
+  void extend(int64_t id, const std::vector<int32_t>& tokens);
+  const StepPlan& schedule_rows(const std::vector<int64_t>& ids, const std::vector<int32_t>& counts,
+                                const std::vector<std::vector<int32_t>>& want);
+  void advance();
+
   // queries
   int num_waiting() const { return static_cast<int>(waiting_.size()); }
   int num_running() const { return static_cast<int>(running_.size()); }

@@ -149,7 +149,13 @@ class LLMEngine:
         sc.max_num_seqs = cfg.max_num_seqs
         sc.max_num_batched_tokens = cfg.max_num_batched_tokens
         sc.max_model_len = self.max_model_len
-        sc.enable_prefix_cache = cfg.enable_prefix_cache
+        # pages can be shared between requests; a recurrent state or carried convolution inputs
+        # cannot be rebuilt from them, so such models recompute every prompt
+        self.stateful = bool(getattr(self.model, "has_sequence_state", False))
+        if self.stateful and cfg.draft_model and cfg.num_speculative_tokens > 0:
+            raise ValueError(f"{self.mcfg.name}: speculative decoding needs a state that rejected drafts can be "
+                             "rolled back from; models with per-sequence recurrent state do not support it")
+        sc.enable_prefix_cache = cfg.enable_prefix_cache and not self.stateful
         sc.chunked_prefill = cfg.chunked_prefill
         sc.cache_threshold = cfg.cache_threshold
         sc.max_prefill_seqs = cfg.max_prefill_seqs
@@ -237,6 +243,8 @@ class LLMEngine:
     # ------------------------------------------------------------------ sizing
     def _block_bytes(self) -> int:
         m = self.mcfg
+        if hasattr(self.model, "cache_bytes_per_block"):
+            return max(1, self.model.cache_bytes_per_block(self.cfg.block_size))
         esz = torch.tensor([], dtype=self.model.dtype).element_size()
         return 2 * m.num_layers * self.model.num_kv_heads_local * self.cfg.block_size * m.head_dim * esz
 
@@ -248,6 +256,8 @@ class LLMEngine:
         m = self.mcfg
         act = self.cfg.max_num_batched_tokens * (6 * m.hidden_size + 4 * m.intermediate_size // max(1, get_state().tp_size)) * 2
         act += self.cfg.max_num_seqs * m.vocab_size * 8 + (2 << 30)
+        if hasattr(self.model, "state_bytes_per_slot"):
+            act += self.cfg.max_num_seqs * self.model.state_bytes_per_slot()
         budget = free - (1.0 - self.cfg.gpu_memory_utilization) * total - act
         n = int(max(64, budget // self._block_bytes()))
         st = get_state()
@@ -731,6 +741,50 @@ class LLMEngine:
         if get_state().tp_size > 1 and self.is_driver:
             comm.tp_broadcast_object(("stop", None), src=0)
 
+    # ------------------------------------------------------------------ teacher-forced replay
+    def score_step(self, entries, end=()) -> Optional[torch.Tensor]:
+        """One teacher-forced step: `entries` = [(request id, its next tokens, offsets among them
+        whose logits are wanted)]; all entries run as one batch from the cache and state that
+        earlier steps left (a request is admitted at its first entry and may sit a step out).
+        `end`: requests finished after this step; their slot and pages go back to the pool.
+        Returns the wanted logits, fp32 [n, V] in the order of the entries (None if n == 0).
+        Nothing is sampled; generation requests must not be mixed into a replaying engine."""
+        if not self.is_driver or get_state().tp_size != 1:
+            raise RuntimeError("score_step runs on a single-rank engine")
+        names = self.__dict__.setdefault("_replay_ids", {})
+        V = self.mcfg.vocab_size
+        ids, counts, wants = [], [], []
+        with self._lock:
+            for rid, toks, want in entries:
+                toks = [int(t) for t in toks]
+                if not toks or min(toks) < 0 or max(toks) >= V:
+                    raise ValueError(f"request {rid!r}: token ids must be in [0, {V}) and not empty")
+                if rid not in names:
+                    names[rid] = next(self._seq_counter)
+                self.sched.extend(names[rid], toks)
+                ids.append(names[rid])
+                counts.append(len(toks))
+                wants.append([int(w) for w in want])
+            plan = self.sched.schedule_rows(ids, counts, wants) if ids else None
+        logits = self.runner.score(plan) if plan is not None else None
+        with self._lock:
+            if plan is not None:
+                self.sched.advance()
+            for rid in end:
+                sid = names.pop(rid, None)
+                if sid is not None:
+                    self.sched.abort(sid)
+        if logits is None:
+            return None
+        # the plan orders its rows (single tokens first); give the logits back in entry order
+        first, k = {}, 0
+        for sid in plan["seq_ids"].tolist():
+            n = len(wants[ids.index(sid)])
+            first[sid] = k
+            k += n
+        order = [first[sid] + j for sid, w in zip(ids, wants) for j in range(len(w))]
+        return logits[torch.tensor(order, dtype=torch.long, device=logits.device)]
+
     # ------------------------------------------------------------------ helpers
     def generate(self, prompts: List[List[int]], params: SamplingParams, max_steps: int = 1 << 30):
         """Blocking batch generation (tests / offline use). Returns output id lists."""
@@ -786,6 +840,8 @@ class LLMEngine:
     def export_prefix(self, tokens: Sequence[int]):
         """CacheEntry for the longest cached page-aligned prefix of `tokens` (this rank's KV shard)."""
         from .kv_io import CacheEntry
+        if self.stateful:
+            raise ValueError("prefix export needs a cache that pages alone describe")
         with self._lock:
             blocks = self.sched.cached_prefix([int(t) for t in tokens])
             idx = torch.tensor(blocks, dtype=torch.long, device=self.device)
@@ -795,6 +851,8 @@ class LLMEngine:
 
     def import_prefix(self, entry) -> int:
         """Install a CacheEntry into the prefix cache; returns #pages newly written."""
+        if self.stateful:
+            raise ValueError("prefix import needs a cache that pages alone describe")
         if entry.block_size != self.cfg.block_size:
             raise ValueError(f"entry block_size {entry.block_size} != engine {self.cfg.block_size}")
         want = tuple(self.runner.kv.shape[:2]) + (entry.kv.shape[2],) + tuple(self.runner.kv.shape[3:])

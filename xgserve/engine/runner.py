@@ -33,6 +33,7 @@ from .. import tune
 from .. import ops
 from ..models.base import AttnMeta
 from ..ops.attention import DecodeWorkspace
+from ..ops.seqmix import SeqMeta
 from ..parallel import comm
 
 # eager (prompt) steps leave their sampled tokens on the device for a looked-ahead successor
@@ -119,16 +120,25 @@ class ModelRunner:
         self.last_logits = None
         cfg = self.cfg
         self.Hkv = model.num_kv_heads_local
-        self.kv = torch.zeros(cfg.num_layers, 2, num_blocks, self.Hkv, block_size, cfg.head_dim,
-                              dtype=self.dtype, device=self.device)
-        self.kv_caches = [(self.kv[i, 0], self.kv[i, 1]) for i in range(cfg.num_layers)]
+        # models with per-sequence state (recurrences, carried convolution inputs) or a cache
+        # layout of their own allocate it themselves: pages + one state row per sequence slot
+        self.seq_state = bool(getattr(model, "has_sequence_state", False))
+        if hasattr(model, "alloc_cache"):
+            self.kv = None
+            self.kv_caches = model.alloc_cache(num_blocks, block_size, max_num_seqs)
+        else:
+            self.kv = torch.zeros(cfg.num_layers, 2, num_blocks, self.Hkv, block_size, cfg.head_dim,
+                                  dtype=self.dtype, device=self.device)
+            self.kv_caches = [(self.kv[i, 0], self.kv[i, 1]) for i in range(cfg.num_layers)]
+        if hasattr(model, "set_max_positions"):
+            model.set_max_positions(max_model_len + 1)
         self.is_cuda = self.device.type == "cuda"
         Hq_local = cfg.num_heads // model.tp
         self.max_splits = tune.get_int("decode_max_splits", 16)
         self.workspace = DecodeWorkspace(max(max_num_seqs, 1), Hq_local, cfg.head_dim, self.max_splits,
-                                         self.device) if self.is_cuda else None
+                                         self.device) if (self.is_cuda and self.kv is not None) else None
         # pinned staging for eager steps
-        cap = 8 * max_num_batched_tokens + 4 * max_num_seqs * (self.max_blocks_per_seq + 4) + 64
+        cap = 9 * max_num_batched_tokens + 4 * max_num_seqs * (self.max_blocks_per_seq + 6) + 64
         # two pinned host staging buffers + device twins: a step may return
         # before its async H2D copy ran, so the next step must not overwrite the
         # same host buffer until that copy's event has completed
@@ -156,7 +166,8 @@ class ModelRunner:
         self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
         # mixed-step graphs: (decode bucket, chunk) -> graph; buckets of >= 16 decode rows
         # whose step stays on the gemm_mw path (decode rows + chunk <= MW_MAX_TOKENS)
-        self.mixed_chunk = int(mixed_chunk) if (self.use_graphs and comm.get_state().tp_size == 1) else 0
+        self.mixed_chunk = int(mixed_chunk) if (self.use_graphs and comm.get_state().tp_size == 1
+                                                and not self.seq_state) else 0
         self.mixed_graphs: Dict[tuple, torch.cuda.CUDAGraph] = {}
         self.mixed_bs: List[int] = []
         self.mixed_replays = 0
@@ -182,6 +193,8 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ utils
     def kv_bytes(self) -> int:
+        if self.kv is None:
+            return self.kv_caches.nbytes()
         return self.kv.numel() * self.kv.element_size()
 
     DECODE_SPLIT_WGS = 512
@@ -203,14 +216,20 @@ class ModelRunner:
         # int32 region: ids | pos | slots | sl | src | bt ; sampling region separate.
         # src[i] >= 0: row i's input id is the previous graph step's sampled token
         # g_out_tok[src[i]] (asynchronous scheduling), substituted inside the graph
-        n = 5 * B + B * W
+        # stateful models: + sslot (the row's state slot, -1 padding) | tseq (its sequence, -1 padding)
+        NS = self.g_nsec = 7 if self.seq_state else 5
+        n = NS * B + B * W
         self.g_int = torch.zeros(n, dtype=torch.int32, device=self.device)
         self.g_ids = self.g_int[0:B]
         self.g_pos = self.g_int[B:2 * B]
         self.g_slot = self.g_int[2 * B:3 * B]
         self.g_sl = self.g_int[3 * B:4 * B]
         self.g_src = self.g_int[4 * B:5 * B]
-        self.g_bt = self.g_int[5 * B:5 * B + B * W].view(B, W)
+        if self.seq_state:
+            self.g_sslot = self.g_int[5 * B:6 * B]
+            self.g_tseq = self.g_int[6 * B:7 * B]
+            self.g_qsl = torch.arange(B + 1, dtype=torch.int32, device=self.device)
+        self.g_bt = self.g_int[NS * B:NS * B + B * W].view(B, W)
         # sampling parameters: one row more than the widest decode graph (mixed steps)
         self.g_temp = torch.zeros(B + 1, dtype=torch.float32, device=self.device)
         self.g_topp = torch.ones(B + 1, dtype=torch.float32, device=self.device)
@@ -254,6 +273,10 @@ class ModelRunner:
         meta = AttnMeta(num_tokens=bs, num_decodes=bs, positions=self.g_pos[:bs], slot_mapping=self.g_slot[:bs],
                         dec_block_tables=self.g_bt[:bs], dec_seq_lens=self.g_sl[:bs],
                         num_splits=self.decode_splits(bs), workspace=self.workspace)
+        if self.seq_state:
+            meta.seq = SeqMeta(num_seqs=bs, max_q=1, qsl=self.g_qsl[:bs + 1], seq_lens=self.g_sl[:bs],
+                               slots=self.g_sslot[:bs], block_tables=self.g_bt[:bs], token_seq=self.g_tseq[:bs],
+                               positions=self.g_pos[:bs], slot_mapping=self.g_slot[:bs])
         h = self.model(self.g_ids[:bs], meta, self.kv_caches)
         logits = self.model.compute_logits(h)
         if greedy:
@@ -315,6 +338,9 @@ class ModelRunner:
         self.g_sl.fill_(0)
         self.g_ids.fill_(0)
         self.g_pos.fill_(0)
+        if self.seq_state:
+            self.g_sslot.fill_(-1)
+            self.g_tseq.fill_(-1)
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
@@ -499,10 +525,16 @@ class ModelRunner:
         hi[4 * B:4 * B + bs] = -1
         if src is not None:
             hi[4 * B:4 * B + n] = src
-        bt = hi[5 * B:5 * B + bs * W].reshape(bs, W)
+        NS = self.g_nsec
+        if self.seq_state:
+            hi[5 * B:5 * B + n] = plan["slots"]
+            hi[5 * B + n:5 * B + bs] = -1
+            hi[6 * B:6 * B + n] = np.arange(n, dtype=np.int32)
+            hi[6 * B + n:6 * B + bs] = -1
+        bt = hi[NS * B:NS * B + bs * W].reshape(bs, W)
         bt[:n, :w] = plan["block_tables"].reshape(n, w)
-        # ids..src (5*B) and the first bs rows of bt: one contiguous H2D copy
-        self.g_int[:5 * B + bs * W].copy_(h_int[:5 * B + bs * W], non_blocking=True)
+        # ids..src (NS*B) and the first bs rows of bt: one contiguous H2D copy
+        self.g_int[:NS * B + bs * W].copy_(h_int[:NS * B + bs * W], non_blocking=True)
         greedy = samp is None or samp.all_greedy
         if not greedy:
             self._stage_sampling(si, samp, n)
@@ -599,7 +631,17 @@ class ModelRunner:
             dev = h_stage
         return dev, np.cumsum([0] + sizes)
 
-    def _execute_eager(self, plan, samp: Optional[SamplingRows], need_hidden: bool, src: Optional[np.ndarray]):
+    @torch.no_grad()
+    def score(self, plan: dict) -> Optional[torch.Tensor]:
+        """Teacher-forced step (StepScheduler.schedule_rows): run the plan's rows through the
+        model and its cache, sample nothing, and return the fp32 logits of the plan's
+        logits_indices rows ([n, V], on the device), or None when it asks for none."""
+        if int(plan["num_tokens"]) == 0:
+            return None
+        return self._execute_eager(plan, None, False, None, score=True)
+
+    def _execute_eager(self, plan, samp: Optional[SamplingRows], need_hidden: bool, src: Optional[np.ndarray],
+                       score: bool = False):
         T = int(plan["num_tokens"])
         Nd = int(plan["num_decodes"])
         ns = int(plan["num_seqs"])
@@ -612,6 +654,10 @@ class ModelRunner:
                  plan["block_tables"], plan["seq_lens"], (qsl[Nd:] - Nd).astype(np.int32), li]
         if src is not None:  # staged with the other inputs: no blocking copy ahead of the queued step
             parts.append(np.ascontiguousarray(src, dtype=np.int32))
+        if self.seq_state:  # the whole step per sequence: first rows, state slots, each token's sequence
+            k_seq = len(parts)
+            parts += [qsl.astype(np.int32), plan["slots"].astype(np.int32),
+                      np.repeat(np.arange(ns, dtype=np.int32), plan["q_lens"])]
         dev, o = self._stage_parts(parts)
         ids = dev[o[0]:o[1]]
         pos = dev[o[1]:o[2]]
@@ -627,8 +673,14 @@ class ModelRunner:
                         num_splits=self.decode_splits(Nd) if self.is_cuda else 1, workspace=self.workspace,
                         pre_block_tables=bt[Nd:], pre_qsl=pre_qsl, pre_seq_lens=sl[Nd:],
                         pre_max_q=int(plan["q_lens"][Nd:].max()) if Np > 0 else 0)
+        if self.seq_state:
+            meta.seq = SeqMeta(num_seqs=ns, max_q=int(plan["max_q_len"]), qsl=dev[o[k_seq]:o[k_seq + 1]],
+                               seq_lens=sl, slots=dev[o[k_seq + 1]:o[k_seq + 2]], block_tables=bt,
+                               token_seq=dev[o[k_seq + 2]:o[k_seq + 3]], positions=pos, slot_mapping=slots)
         h = self.model(ids, meta, self.kv_caches)
         hid = h if need_hidden else None
+        if score:
+            return self.model.compute_logits(h.index_select(0, lidx.long())).float() if S else None
         if S == 0:
             return (0, hid, (np.zeros(0, np.int32), np.zeros(0, np.float32), hid), None)
         logits = self.model.compute_logits(h.index_select(0, lidx.long()))

@@ -30,6 +30,8 @@ class AttnMeta:
     pre_qsl: Optional[torch.Tensor] = None
     pre_seq_lens: Optional[torch.Tensor] = None
     pre_max_q: int = 0
+    # per-sequence view of the whole step (ops.seqmix.SeqMeta): models with per-slot state
+    seq: Optional[object] = None
 
     @property
     def num_prefill_tokens(self) -> int:

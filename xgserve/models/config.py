@@ -16,7 +16,7 @@ from typing import Dict, List, Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                      # "llama" | "mixtral" | "gpt2"
+    arch: str                      # "llama" | "mixtral" | "gpt2" | "dofivik"
     hidden_size: int
     num_layers: int
     num_heads: int
@@ -34,6 +34,11 @@ class ModelConfig:
     bos_token_id: int = 1
     eos_token_ids: List[int] = field(default_factory=lambda: [2])
     dtype: str = "bfloat16"
+    # layer-list architectures ("dofivik"): one dict per layer {"type", "mixer", "mlp"}, the
+    # residual scale of the norm-after-sum sublayers, and the taps of the input convolution
+    layer_specs: Optional[List[dict]] = None
+    postln_alpha: float = 1.0
+    canon_taps: int = 1
 
     @property
     def q_size(self) -> int:
@@ -45,6 +50,9 @@ class ModelConfig:
 
     def num_params(self) -> int:
         H, F, V, L = self.hidden_size, self.intermediate_size, self.vocab_size, self.num_layers
+        if self.layer_specs is not None:
+            from .dofivik import count_params
+            return count_params(self)
         attn = H * (self.q_size + 2 * self.kv_size) + self.q_size * H
         if self.arch == "mixtral":
             mlp = self.num_experts * 3 * H * F + H * self.num_experts
@@ -56,6 +64,9 @@ class ModelConfig:
         return L * (attn + mlp + 2 * H) + emb + H
 
     def kv_bytes_per_token(self, tp: int = 1, dtype_bytes: int = 2) -> int:
+        if self.layer_specs is not None:
+            return sum((m["kv_rank"] + m["rot_dim"]) * dtype_bytes for m in (L["mixer"] for L in self.layer_specs)
+                       if "kv_rank" in m and "kv_from" not in m)
         kvh = max(1, self.num_kv_heads // tp)
         return 2 * self.num_layers * kvh * self.head_dim * dtype_bytes
 
@@ -92,6 +103,44 @@ register(ModelConfig("llama-tiny-gqa8", "llama", 512, 2, 8, 8, 64, 1024, 512, 10
                      bos_token_id=1, eos_token_ids=[2]))
 register(ModelConfig("mixtral-tiny", "mixtral", 256, 2, 4, 2, 64, 256, 512, 1024, 1000000.0,
                      num_experts=8, experts_per_token=2, bos_token_id=1, eos_token_ids=[2]))
+
+
+def dofivik_config(name: str, width: int, vocab: int, layers: List[dict], postln_alpha: float = 2.0, taps: int = 4,
+                   eps: float = 1e-6, max_position: int = 32768) -> ModelConfig:
+    """A Dofivik model: a list of layers, each one mixer ("latent_attention": sliding-window attention
+    over a cached low-rank latent + one shared rotary key; "general_delta": a generalized delta-rule
+    recurrence) and an optional dense xIELU feed-forward, every sublayer reading h + conv(h) and
+    followed by the norm of alpha * x + sublayer(x)."""
+    att = [L["mixer"] for L in layers if L["type"] == "latent_attention"]
+    heads = max([L["mixer"]["heads"] for L in layers] or [1])
+    hd = max([m["dim"] + m["rot_dim"] for m in att] or [L["mixer"]["dim"] for L in layers] or [1])
+    ff = max([L["mlp"]["ff"] for L in layers if L.get("mlp")] or [0])
+    for i, L in enumerate(layers):
+        if L["type"] not in ("latent_attention", "general_delta"):
+            raise ValueError(f"layer {i}: unknown mixer type {L['type']!r}")
+        if L.get("mlp") is not None and L["mlp"].get("kind", "dense") != "dense":
+            raise ValueError(f"layer {i}: unknown feed-forward kind {L['mlp'].get('kind')!r}")
+        src = L["mixer"].get("kv_from")
+        if src is not None:
+            m, o = L["mixer"], (layers[src]["mixer"] if 0 <= src < i else None)
+            if o is None or layers[src]["type"] != "latent_attention" or "kv_from" in o:
+                raise ValueError(f"layer {i}: kv_from must name an earlier latent_attention layer with its own cache")
+            if (o["kv_rank"], o["rot_dim"], o["rot"]) != (m["kv_rank"], m["rot_dim"], m["rot"]):
+                raise ValueError(f"layer {i}: kv_from layer {src} has another latent size or rotation")
+    return ModelConfig(name, "dofivik", width, len(layers), heads, 1, hd, ff, vocab, max_position, 0.0, None, eps,
+                       False, bos_token_id=0, eos_token_ids=[], layer_specs=layers, postln_alpha=float(postln_alpha),
+                       canon_taps=int(taps))
+
+
+def _dofivik_tiny_layers():
+    att = {"dim": 32, "heads": 4, "kv_rank": 48, "q_rank": 40, "rot_dim": 16, "vdim": 24, "scale": 48 ** -0.5,
+           "mask": {"size": 24}, "rot": {"base": 10000.0, "dims": 16}}
+    return [{"type": "latent_attention", "mixer": dict(att), "mlp": {"kind": "dense", "ff": 192}},
+            {"type": "general_delta", "mixer": {"dim": 32, "heads": 4}, "mlp": None},
+            {"type": "latent_attention", "mixer": dict(att, kv_from=0), "mlp": {"kind": "dense", "ff": 192}}]
+
+
+register(dofivik_config("dofivik-tiny", 128, 512, _dofivik_tiny_layers(), max_position=1024))
 register(ModelConfig("gpt2-tiny", "gpt2", 128, 2, 2, 2, 64, 512, 512, 256, 0.0, tie_embeddings=True,
                      bos_token_id=0, eos_token_ids=[0], dtype="float32"))
 
@@ -111,6 +160,9 @@ def list_models() -> List[str]:
 def from_hf_config(path: str, name: Optional[str] = None) -> ModelConfig:
     with open(path) as f:
         c = json.load(f)
+    if c.get("architecture") == "Dofivik":
+        return dofivik_config(name or "dofivik", c["width"], c["vocab"], c["layers"], c["postln_alpha"],
+                              c["canon"]["taps"], c["norm"]["eps"], int(c.get("max_position", 32768)))
     mt = c.get("model_type", "llama")
     eos = c.get("eos_token_id", 2)
     eos = eos if isinstance(eos, list) else [eos]

@@ -19,12 +19,23 @@ import torch
 from ..ops.linear import deinterleave_gate_up, interleave_gate_up
 from .base import kv_head_range
 from .config import ModelConfig, get_config
+from .dofivik import DofivikForCausalLM
 from .gpt2 import GPT2ForCausalLM
 from .llama import LlamaForCausalLM
 
 
 def model_class(cfg: ModelConfig):
-    return GPT2ForCausalLM if cfg.arch == "gpt2" else LlamaForCausalLM
+    return {"gpt2": GPT2ForCausalLM, "dofivik": DofivikForCausalLM}.get(cfg.arch, LlamaForCausalLM)
+
+
+def _resolve_shapes(cfg: ModelConfig, checkpoint: str) -> None:
+    """Sizes that only a tensor's shape gives (Dofivik: the rank of the decay projection)."""
+    if cfg.arch != "dofivik":
+        return
+    r = _Reader(checkpoint)
+    for i, spec in enumerate(cfg.layer_specs):
+        if spec["type"] == "general_delta":
+            spec["mixer"]["decay_rank"] = int(r.shape(f"l{i}.mix.w1")[0])
 
 
 def build_model(cfg: ModelConfig, device="cpu", dtype: Optional[torch.dtype] = None,
@@ -35,6 +46,8 @@ def build_model(cfg: ModelConfig, device="cpu", dtype: Optional[torch.dtype] = N
     everything else stay `dtype`."""
     if dtype is None:
         dtype = torch.float32 if (cfg.dtype == "float32" and torch.device(device).type == "cpu") else torch.bfloat16
+    if checkpoint:
+        _resolve_shapes(cfg, checkpoint)
     m = model_class(cfg)(cfg, device=device, dtype=dtype, tp=tp, rank=rank)
     if checkpoint:
         load_checkpoint(m, checkpoint)
@@ -75,6 +88,11 @@ class _Reader:
     def has(self, name: str) -> bool:
         return name in self.where
 
+    def shape(self, name: str):
+        if name not in self.where:
+            raise KeyError(f"missing tensor {name!r} in checkpoint {self.path}")
+        return tuple(self.handles[self.where[name]].get_slice(name).get_shape())
+
     def get(self, name: str, dim: Optional[int] = None, start: int = 0, length: Optional[int] = None) -> torch.Tensor:
         if name not in self.where:
             raise KeyError(f"missing tensor {name!r} in checkpoint {self.path}")
@@ -100,6 +118,8 @@ def load_checkpoint(model, path: str) -> None:
     cfg = model.cfg
     if cfg.arch == "gpt2":
         _load_gpt2(model, r)
+    elif cfg.arch == "dofivik":
+        _load_dofivik(model, r)
     else:
         _load_llama(model, r)
 
@@ -173,6 +193,62 @@ def _load_gpt2(m, r: _Reader):
         _copy(L.proj_b, r.get(b + "mlp.c_proj.bias"), "mlp.c_proj.b")
 
 
+def _dofivik_tensors(m):
+    """(checkpoint name, parameter, row range of a fused parameter or None) for every tensor."""
+    out = [("embed", m.embed, None), ("head", m.head, None), ("final.norm", m.final_norm, None)]
+    for i, L in enumerate(m.layers):
+        b, x = f"l{i}.", L.mix
+        out += [(b + "norm1", L.norm1, None), (b + "canon1", L.canon1, None)]
+        if L.kind == "latent_attention":
+            out += [(b + "mix.dq", x.in_proj, (0, x.Rq)), (b + "mix.dq.norm", x.q_norm, None),
+                    (b + "mix.g", x.in_proj, (x.off_g, x.off_g + x.H)), (b + "mix.uq", x.uq, None),
+                    (b + "mix.uk", x.uk, None), (b + "mix.uv", x.uv, None), (b + "mix.o", x.o, None)]
+            if x.own_kv:
+                out += [(b + "mix.dkv", x.in_proj, (x.off_kv, x.off_kv + x.R + x.rd)), (b + "mix.dkv.norm", x.kv_norm, None)]
+        else:
+            HD = x.HD
+            for j, n in enumerate(("r", "k", "v", "g", "a")):
+                out.append((b + "mix." + n, x.in_proj, (j * HD, (j + 1) * HD)))
+            out += [(b + "mix.w1", x.in_proj, (5 * HD, 5 * HD + x.lr)), (b + "mix.w2", x.w2, None),
+                    (b + "mix.w0", x.w0, None), (b + "mix.a.b", x.a_bias, None), (b + "mix.norm", x.norm, None),
+                    (b + "mix.o", x.o, None)]
+        if L.mlp is not None:
+            out += [(b + "norm2", L.norm2, None), (b + "canon2", L.canon2, None), (b + "mlp.up", L.mlp.up, None),
+                    (b + "mlp.up.b", L.mlp.up_b, None), (b + "mlp.down", L.mlp.down, None),
+                    (b + "mlp.down.b", L.mlp.down_b, None), (b + "mlp.act", L.mlp.act, None)]
+    return out
+
+
+def _load_dofivik(m, r: _Reader):
+    """Tensors `l<i>.<norm1|norm2|canon1|canon2>`, `l<i>.mix.*`, `l<i>.mlp.*`, `embed`, `final.norm`, `head`
+    ([out, in] matrices); the projections that read the same input are fused row-wise on load."""
+    for name, p, rows in _dofivik_tensors(m):
+        src = r.get(name)
+        dst = p.data if rows is None else p.data[rows[0]:rows[1]]
+        if tuple(dst.shape) != tuple(src.shape):
+            raise ValueError(f"shape mismatch for {name}: model {tuple(dst.shape)} vs checkpoint {tuple(src.shape)}")
+        dst.copy_(src.to(dst.dtype))
+    m.finalize_weights()
+
+
+def _save_dofivik(model, path: str) -> None:
+    from safetensors.torch import save_file
+    cfg = model.cfg
+    t = {}
+    for name, p, rows in _dofivik_tensors(model):
+        v = p.data if rows is None else p.data[rows[0]:rows[1]]
+        t[name] = v.detach().to(torch.bfloat16).contiguous().cpu()
+    save_file(t, os.path.join(path, "model.safetensors"))
+    layers = []
+    for spec in cfg.layer_specs:
+        mx = {k: v for k, v in spec["mixer"].items() if k != "decay_rank"}
+        layers.append({"type": spec["type"], "mixer": mx, "mlp": spec.get("mlp")})
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump({"architecture": "Dofivik", "width": cfg.hidden_size, "vocab": cfg.vocab_size, "layers": layers,
+                   "postln_alpha": cfg.postln_alpha, "canon": {"taps": cfg.canon_taps},
+                   "norm": {"eps": cfg.norm_eps}}, f, indent=1)
+
+
 @torch.no_grad()
 def save_checkpoint(model, path: str) -> None:
     """Write a TP=1 model in HF layout (safetensors + config.json)."""
@@ -180,6 +256,8 @@ def save_checkpoint(model, path: str) -> None:
     assert model.tp == 1, "save from a TP=1 model"
     cfg = model.cfg
     os.makedirs(path, exist_ok=True)
+    if cfg.arch == "dofivik":
+        return _save_dofivik(model, path)
     t: Dict[str, torch.Tensor] = {}
     if cfg.arch == "gpt2":
         t["transformer.wte.weight"] = model.wte

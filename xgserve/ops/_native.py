@@ -38,6 +38,35 @@ def kernels():
             f"{e!r}. Run `python -m xgserve._build`.") from e
 
 
+_M = None
+
+
+def mixers():
+    """The sequence-mixer kernel library (xgserve._mixers: csrc/mixers); raises if it is not built."""
+    global _M
+    if _M is None:
+        try:
+            from .. import _mixers as m  # noqa: WPS433
+        except Exception as e:  # pragma: no cover - depends on build
+            raise RuntimeError("xgserve._mixers (HIP/gfx950) is not built or failed to load: "
+                               f"{e!r}. Run `python -m xgserve._build --only mixers`.") from e
+        _M = m
+    return _M
+
+
+def native_device(t: torch.Tensor) -> bool:
+    """True when `t` lives on the GPU: its ops run on the HIP kernels or raise."""
+    return t.device.type == "cuda"
+
+
+def is_f32(t: torch.Tensor) -> bool:
+    if t.dtype == torch.float32:
+        return True
+    if t.dtype == torch.bfloat16:
+        return False
+    raise TypeError(f"activations must be float32 or bfloat16, got {t.dtype}")
+
+
 def available() -> bool:
     try:
         kernels()

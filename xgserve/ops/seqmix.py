@@ -1,0 +1,306 @@
+"""Operators of the stateful / latent-cache decoder layers (csrc/mixers).
+
+A ragged step is described by a `SeqMeta`: per sequence its first row (`qsl`), the
+tokens it holds after the step (`seq_lens`), its state row (`slots`, < 0: padding) and
+its page table; per token its position, cache row (`slot_mapping`) and sequence
+(`token_seq`). A sequence with an empty context starts from zero state whatever its
+slot holds. GPU tensors run on the HIP kernels; CPU tensors on the PyTorch forms below
+(the same paged / carried semantics, used by the CPU engine).
+
+The residual stream, norms, softmax, rotations and recurrences are fp32; `act` tensors
+(GEMM inputs / outputs, caches) are bfloat16 or float32.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from ._native import is_f32, mixers, native_device, stream_ptr
+
+
+@dataclass
+class SeqMeta:
+    num_seqs: int
+    max_q: int
+    qsl: torch.Tensor            # int32 [num_seqs + 1]
+    seq_lens: torch.Tensor       # int32 [num_seqs]
+    slots: torch.Tensor          # int32 [num_seqs]
+    block_tables: torch.Tensor   # int32 [num_seqs, width]
+    token_seq: torch.Tensor      # int32 [T]
+    positions: torch.Tensor      # int32 [T]
+    slot_mapping: torch.Tensor   # int32 [T]
+
+
+def _p(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def _i32(t: torch.Tensor) -> torch.Tensor:
+    assert t.dtype == torch.int32 and t.is_contiguous()
+    return t
+
+
+# ---------------------------------------------------------------------------- embedding
+def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """fp32 rows table[ids] (zero rows for ids outside the table)."""
+    V, W = table.shape
+    if not native_device(table):
+        ok = (ids >= 0) & (ids < V)
+        out = table[ids.long().clamp(0, V - 1)].float()
+        out[~ok] = 0
+        return out
+    out = torch.empty(ids.shape[0], W, dtype=torch.float32, device=table.device)
+    mixers().embed_rows(_i32(ids).data_ptr(), table.data_ptr(), is_f32(table), out.data_ptr(), ids.shape[0], W, V,
+                        stream_ptr())
+    return out
+
+
+# ---------------------------------------------------------------------------- input convolution
+def causal_conv_residual(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor, sm: SeqMeta,
+                         out_dtype: torch.dtype) -> torch.Tensor:
+    """h + conv(h) per channel over time: out_t = x_t + sum_j w[:, j] x_(t - taps + 1 + j), zeros
+    before a sequence's start. x fp32 [T, W]; w fp32 [W, taps]; state fp32 [slots, taps - 1, W]
+    holds each sequence's last taps - 1 inputs and is updated."""
+    T, W = x.shape
+    taps = w.shape[1]
+    out = torch.empty(T, W, dtype=out_dtype, device=x.device)
+    if native_device(x):
+        assert x.dtype == torch.float32 and x.is_contiguous() and w.dtype == torch.float32 and w.is_contiguous()
+        assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (taps - 1, W)
+        mixers().canon_conv(x.data_ptr(), w.data_ptr(), state.data_ptr(), _i32(sm.qsl).data_ptr(),
+                            _i32(sm.seq_lens).data_ptr(), _i32(sm.slots).data_ptr(), out.data_ptr(), is_f32(out),
+                            sm.num_seqs, sm.max_q, W, taps, stream_ptr())
+        return out
+    nh = taps - 1
+    qsl, sl, slots = sm.qsl.tolist(), sm.seq_lens.tolist(), sm.slots.tolist()
+    for s in range(sm.num_seqs):
+        a, b = qsl[s], qsl[s + 1]
+        if slots[s] < 0 or b <= a:
+            continue
+        ctx = sl[s] - (b - a)
+        hist = state[slots[s]] if ctx > 0 else torch.zeros(nh, W)
+        ext = torch.cat([hist, x[a:b]], 0)
+        y = x[a:b].clone()
+        for j in range(taps):
+            y += w[:, j] * ext[j:j + b - a]
+        out[a:b] = y.to(out_dtype)
+        if nh:
+            state[slots[s]] = ext[-nh:]
+    return out
+
+
+# ---------------------------------------------------------------------------- norm after the sum
+def scaled_add_rmsnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: torch.Tensor, eps: float, alpha: float = 1.0,
+                       bias: Optional[torch.Tensor] = None, w_offset: float = 0.0, inplace: bool = True,
+                       out_dtype: Optional[torch.dtype] = None):
+    """v = alpha * x + y + bias; r = v / sqrt(mean(v^2) + eps) * (w_offset + w), in fp32.
+    x fp32 [T, W] (overwritten with r when `inplace`); y an activation tensor or None.
+    Returns r as fp32 (inplace) or as `out_dtype`."""
+    T, W = x.shape
+    if not native_device(x):
+        v = alpha * x
+        if y is not None:
+            v = v + y.float()
+        if bias is not None:
+            v = v + bias
+        r = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * (w_offset + w)
+        if inplace:
+            x.copy_(r)
+            return x
+        return r.to(out_dtype or torch.float32)
+    assert x.dtype == torch.float32 and x.is_contiguous() and w.dtype == torch.float32
+    out = None if inplace else torch.empty(T, W, dtype=out_dtype or torch.float32, device=x.device)
+    if y is not None:
+        assert y.stride(-1) == 1 and y.shape == x.shape
+    mixers().scaled_add_rmsnorm(x.data_ptr(), _p(y), is_f32(y) if y is not None else True,
+                                y.stride(0) if y is not None else 0, _p(bias), float(alpha), w.data_ptr(),
+                                float(w_offset), float(eps), x.data_ptr() if inplace else 0, _p(out),
+                                is_f32(out) if out is not None else True, T, W, stream_ptr())
+    return x if inplace else out
+
+
+# ---------------------------------------------------------------------------- rotation table
+def build_rot_table(dims: int, base: float, max_pos: int, device="cpu") -> torch.Tensor:
+    """fp32 [max_pos, dims / 2, 2] = (cos, sin) of position * base^(-2 i / dims): the angles of the
+    interleaved-pair rotation (dimension 2i with 2i + 1), evaluated in fp64."""
+    inv = base ** (-torch.arange(0, dims, 2, dtype=torch.float64) / dims)
+    ang = torch.outer(torch.arange(max_pos, dtype=torch.float64), inv)
+    return torch.stack([ang.cos(), ang.sin()], -1).float().contiguous().to(device)
+
+
+def _rotate_pairs(v: torch.Tensor, rot: torch.Tensor, pos: torch.Tensor, dims: int) -> torch.Tensor:
+    """v [T, ..., n] fp32: rotate the first `dims` entries pairwise by the table rows of `pos`."""
+    cs = rot[pos.long()]  # [T, dims/2, 2]
+    while cs.dim() < v.dim() + 1:
+        cs = cs.unsqueeze(1)
+    c, s = cs[..., 0], cs[..., 1]
+    a, b = v[..., 0:dims:2], v[..., 1:dims:2]
+    out = v.clone()
+    out[..., 0:dims:2] = a * c - b * s
+    out[..., 1:dims:2] = b * c + a * s
+    return out
+
+
+# ---------------------------------------------------------------------------- latent attention
+def latent_prep(proj: torch.Tensor, off_q: int, Rq: int, off_kv: int, R: int, rd: int, wq: torch.Tensor,
+                wkv: Optional[torch.Tensor], eps: float, rot: torch.Tensor, rot_dims: int, sm: SeqMeta,
+                cache: Optional[torch.Tensor]) -> torch.Tensor:
+    """From a fused projection row: the query latent (RMS-normed, weight wq) is returned; with
+    off_kv >= 0 the key/value latent (RMS-normed, weight wkv) and the shared rotary key (rotated by
+    its position) are written to cache row slot_mapping[t] as [latent (R) | key (rd)]."""
+    T = proj.shape[0]
+    cq = torch.empty(T, Rq, dtype=proj.dtype, device=proj.device)
+    if native_device(proj):
+        assert proj.stride(1) == 1 and rot.dtype == torch.float32
+        if off_kv >= 0:
+            assert cache.is_contiguous() and cache.dtype == proj.dtype and cache.shape[-1] == R + rd
+        mixers().latent_prep(proj.data_ptr(), is_f32(proj), proj.stride(0), off_q, Rq, off_kv, R, rd, wq.data_ptr(),
+                             _p(wkv), float(eps), _i32(sm.positions).data_ptr(), _i32(sm.slot_mapping).data_ptr(),
+                             rot.data_ptr(), rot_dims, cq.data_ptr(), _p(cache) if off_kv >= 0 else 0, T, stream_ptr())
+        return cq
+    pf = proj.float()
+    v = pf[:, off_q:off_q + Rq]
+    cq.copy_((v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * wq).to(proj.dtype))
+    if off_kv >= 0:
+        c = pf[:, off_kv:off_kv + R]
+        c = c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + eps) * wkv
+        kr = _rotate_pairs(pf[:, off_kv + R:off_kv + R + rd], rot, sm.positions, rot_dims)
+        rows = torch.cat([c, kr], -1).to(cache.dtype)
+        ok = sm.slot_mapping >= 0
+        cache.view(-1, R + rd)[sm.slot_mapping[ok].long()] = rows[ok]
+    return cq
+
+
+def latent_attention(qabs: torch.Tensor, q: torch.Tensor, dn: int, gate: torch.Tensor, cache: torch.Tensor,
+                     rot: torch.Tensor, rot_dims: int, window: int, scale: float, block_size: int,
+                     sm: SeqMeta) -> torch.Tensor:
+    """Sliding-window softmax attention in latent space. Every head scores the same cached rows
+    [latent (R) | rotated key (rd)]: head h of token t uses qabs[h, t] (its unrotated query mapped into
+    latent space) and the rotary part q[t, h, dn:], rotated here; the output is the softmax-weighted
+    mean of the latents, times sigmoid(gate[t, h]). Position i sees j with 0 <= i - j < window.
+    qabs [H, T, R]; q [T, H, dn + rd]; gate [T, >= H] (row-strided); returns [H, T, R]."""
+    H, T, R = qabs.shape
+    dq = q.shape[-1]
+    rd = dq - dn
+    out = torch.empty(H, T, R, dtype=qabs.dtype, device=qabs.device)
+    if native_device(qabs):
+        assert qabs.is_contiguous() and q.is_contiguous() and cache.is_contiguous() and gate.stride(1) == 1
+        assert cache.dtype == qabs.dtype == q.dtype == gate.dtype and cache.shape[-1] == R + rd
+        bt = _i32(sm.block_tables)
+        mixers().latent_attention(qabs.data_ptr(), q.data_ptr(), is_f32(q), H * dq, dq, dn, gate.data_ptr(),
+                                  gate.stride(0), cache.data_ptr(), bt.data_ptr(), bt.shape[1], block_size,
+                                  _i32(sm.positions).data_ptr(), _i32(sm.token_seq).data_ptr(), rot.data_ptr(), rot_dims,
+                                  out.data_ptr(), T, H, R, rd, int(window), float(scale), stream_ptr())
+        return out
+    rows = cache.view(-1, R + rd)
+    qr = _rotate_pairs(q.float()[..., dn:], rot, sm.positions, rot_dims)  # [T, H, rd]
+    qa = qabs.float()
+    tseq, pos = sm.token_seq.tolist(), sm.positions.tolist()
+    for t in range(T):
+        s = tseq[t]
+        if s < 0:
+            out[:, t] = 0
+            continue
+        j0 = max(0, pos[t] - window + 1)
+        keys = torch.arange(j0, pos[t] + 1)
+        idx = sm.block_tables[s][(keys // block_size).long()].long() * block_size + keys % block_size
+        kv = rows[idx].float()  # [n, R + rd]
+        sc = (qa[:, t] @ kv[:, :R].T + qr[t] @ kv[:, R:].T) * scale
+        p = torch.softmax(sc, -1)
+        out[:, t] = ((p @ kv[:, :R]) * torch.sigmoid(gate[t, :H].float())[:, None]).to(out.dtype)
+    return out
+
+
+def heads_to_rows(x: torch.Tensor) -> torch.Tensor:
+    """[H, T, n] -> [T, H * n]."""
+    H, T, n = x.shape
+    if not native_device(x):
+        return x.transpose(0, 1).reshape(T, H * n)
+    out = torch.empty(T, H * n, dtype=x.dtype, device=x.device)
+    mixers().heads_to_rows(x.contiguous().data_ptr(), is_f32(x), out.data_ptr(), T, H, n, stream_ptr())
+    return out
+
+
+# ---------------------------------------------------------------------------- generalized delta rule
+DECAY_SCALE = math.exp(-0.5)
+UNIT_KEY_EPS = 1e-6
+
+
+def delta_rule_scan(proj: torch.Tensor, off_r: int, off_k: int, off_v: int, off_a: int, wl: torch.Tensor,
+                    a_bias: torch.Tensor, w0: torch.Tensor, state: torch.Tensor, H: int, D: int,
+                    sm: SeqMeta) -> torch.Tensor:
+    """Per head, with r, k, v, a-logits at column offsets of the fused projection row and the decay
+    logits wl [T, H * D]:  w = exp(-e^(-1/2) sigmoid(wl + w0)), a = sigmoid(a_logit + a_bias),
+    u = k / sqrt(|k|^2 + 1e-6);  S <- diag(w) S - (a u)(u^T S) + k v^T (both read the old S);
+    o = S^T r. state fp32 [slots, H, D, D] is carried and updated. Returns o fp32 [T, H * D]."""
+    T = proj.shape[0]
+    o = torch.empty(T, H * D, dtype=torch.float32, device=proj.device)
+    if native_device(proj):
+        assert proj.stride(1) == 1 and wl.stride(1) == 1 and wl.dtype == proj.dtype
+        assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, D, D)
+        mixers().delta_scan(proj.data_ptr(), is_f32(proj), proj.stride(0), off_r, off_k, off_v, off_a, wl.data_ptr(),
+                            wl.stride(0), a_bias.data_ptr(), w0.data_ptr(), state.data_ptr(), _i32(sm.qsl).data_ptr(),
+                            _i32(sm.seq_lens).data_ptr(), _i32(sm.slots).data_ptr(), o.data_ptr(), sm.num_seqs, H, D,
+                            stream_ptr())
+        return o
+    pf = proj.float()
+    HD = H * D
+    r, k, v = (pf[:, off:off + HD].view(T, H, D) for off in (off_r, off_k, off_v))
+    a = torch.sigmoid(pf[:, off_a:off_a + HD] + a_bias).view(T, H, D)
+    w = torch.exp(-DECAY_SCALE * torch.sigmoid(wl.float() + w0)).view(T, H, D)
+    u = k / torch.sqrt(k.pow(2).sum(-1, keepdim=True) + UNIT_KEY_EPS)
+    qsl, sl, slots = sm.qsl.tolist(), sm.seq_lens.tolist(), sm.slots.tolist()
+    for s in range(sm.num_seqs):
+        lo, hi = qsl[s], qsl[s + 1]
+        if slots[s] < 0 or hi <= lo:
+            continue
+        S = state[slots[s]].clone() if sl[s] - (hi - lo) > 0 else torch.zeros(H, D, D)
+        for t in range(lo, hi):
+            uS = torch.einsum("hi,hij->hj", u[t], S)
+            S = w[t][:, :, None] * S - (a[t] * u[t])[:, :, None] * uS[:, None, :] + k[t][:, :, None] * v[t][:, None, :]
+            o[t] = torch.einsum("hij,hi->hj", S, r[t]).reshape(HD)
+        state[slots[s]] = S
+    return o
+
+
+def delta_rule_out(o: torch.Tensor, norm_w: torch.Tensor, gate: torch.Tensor, eps: float, H: int, D: int,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """Each head's o / rms(o), times norm_w, times sigmoid(gate). o fp32 [T, H * D]; gate [T, H * D] (row-strided)."""
+    T = o.shape[0]
+    if not native_device(o):
+        v = o.view(T, H, D)
+        v = (v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, H * D)
+        return (v * norm_w * torch.sigmoid(gate.float())).to(out_dtype)
+    out = torch.empty(T, H * D, dtype=out_dtype, device=o.device)
+    assert gate.stride(1) == 1 and gate.dtype == out_dtype
+    mixers().delta_out(o.data_ptr(), norm_w.data_ptr(), gate.data_ptr(), is_f32(gate), gate.stride(0), float(eps),
+                       out.data_ptr(), T, H, D, stream_ptr())
+    return out
+
+
+# ---------------------------------------------------------------------------- activations
+def xielu(z: torch.Tensor, bias: Optional[torch.Tensor], sp: float, cn: float) -> torch.Tensor:
+    """xIELU of z + bias with sp = softplus(p), cn = 1/2 + softplus(q):
+    z > 0: sp z^2 + z / 2;  z <= 0: cn (exp(z) - 1 - z) + z / 2."""
+    if not native_device(z):
+        v = z.float() + (bias if bias is not None else 0)
+        neg = cn * (torch.expm1(v.clamp(max=0)) - v) + 0.5 * v
+        return torch.where(v > 0, sp * v * v + 0.5 * v, neg).to(z.dtype)
+    assert z.is_contiguous()
+    out = torch.empty_like(z)
+    mixers().xielu(z.data_ptr(), is_f32(z), _p(bias), float(sp), float(cn), out.data_ptr(), z.numel(), z.shape[-1],
+                   stream_ptr())
+    return out
+
+
+def tanh_cols(x: torch.Tensor, off: int, n: int) -> torch.Tensor:
+    """tanh of columns [off, off + n) of a row-strided activation tensor, as a contiguous [T, n]."""
+    T = x.shape[0]
+    if not native_device(x):
+        return torch.tanh(x[:, off:off + n].float()).to(x.dtype)
+    out = torch.empty(T, n, dtype=x.dtype, device=x.device)
+    mixers().tanh_cols(x.data_ptr() + off * x.element_size(), is_f32(x), x.stride(0), out.data_ptr(), T, n, stream_ptr())
+    return out
