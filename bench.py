@@ -65,6 +65,14 @@ def parse():
                     help="single-GPU simulation of ONE rank of a TP group of this degree: the rank's weight / "
                          "KV shards and kernels, collectives replaced by local reductions (not a TP measurement: "
                          "xGMI time is excluded; reported with parallelism 'tpN-shard-sim')")
+    ap.add_argument("--dofivik", action="store_true",
+                    help="instead of the headline: prefill and decode tokens/s of Dofivik beside a Llama of equal "
+                         "layer sizes (bench/dofivik_bench.py; --prompt-len, --concurrency = decode batch, --steps, "
+                         "--warmup apply)")
+    ap.add_argument("--dofivik-sizes", default="1b-class,8b-class")
+    ap.add_argument("--dofivik-prompts", type=int, default=4, help="prompts in the one prefill step")
+    ap.add_argument("--dofivik-context", type=int, default=1024, help="context length of the decoding rows")
+    ap.add_argument("--dofivik-only", default=None, choices=["dofivik", "llama"])
     return ap.parse_args()
 
 
@@ -159,6 +167,14 @@ def preflight(st, world: int, tp: int, dev, eng) -> dict:
 
 def main():
     a = parse()
+    if a.dofivik:
+        import importlib.util
+        here = os.path.dirname(os.path.abspath(__file__))
+        sys.path.insert(0, here)
+        spec = importlib.util.spec_from_file_location("dofivik_bench", os.path.join(here, "bench", "dofivik_bench.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        return mod.run(a)
     env_world = os.environ.get("WORLD_SIZE")
     if env_world is None and a.gpus > 1:
         return launch_ranks(a.gpus)
