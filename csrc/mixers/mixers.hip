@@ -314,6 +314,168 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
   }
 }
 
+// ---- MFMA form (bf16 activations / cache; R % 16 == 0, rd % 8 == 0)
+// One wave = 16 query slots: 16 tokens of one head (prompt portions) or one token of up to
+// 16 heads (single-token rows); a workgroup's 4 waves take 4 heads (or head tiles) of the same
+// tokens and share each staged tile of 64 cached rows. S^T = K . Q^T on
+// v_mfma_f32_16x16x32_bf16 (a lane owns one query's scores), whose accumulator is, packed,
+// the B operand of O^T += V^T . P^T; V^T fragments are transposed LDS reads of the same tile.
+constexpr int kKT = 64;
+
+template <int NMT_MAX>
+__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
+    const bf16* __restrict__ qabs, const bf16* __restrict__ q, int dq, int dn, const bf16* __restrict__ gate,
+    int64_t gate_stride, const bf16* __restrict__ cache, const int32_t* __restrict__ block_tables, int bt_width, int bs,
+    const int32_t* __restrict__ qsl, const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots,
+    const float* __restrict__ rot, int rot_dims, bf16* __restrict__ out, int Ttot, int H, int R, int rd, int window,
+    float scale, int TPT, int HPT) {
+  constexpr int NKK_MAX = NMT_MAX / 2 + 4;
+  extern __shared__ __attribute__((aligned(16))) uint16_t tile_lds[];
+  const int Dk = R + rd, nkk = (Dk + 31) >> 5, nmt = R >> 4, LDK = nkk * 32 + 8;
+  const int s = blockIdx.y;
+  const int q0 = qsl[s], qn = qsl[s + 1] - q0;
+  if (slots[s] < 0 || qn <= 0) return;
+  const int t0 = blockIdx.x * TPT;
+  if (t0 >= qn) return;
+  const int ctx = seq_lens[s] - qn;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int li = lane & 15, g = lane >> 4;
+  const int h0 = (blockIdx.z * 4 + wave) * HPT;
+  const bool wave_on = h0 < H;
+  const int tl = li / HPT, head = h0 + li % HPT, tok = t0 + tl;
+  const bool valid = wave_on && tl < TPT && tok < qn && head < H;
+  const int pos_q = ctx + tok;
+  const int pos_last = ctx + min(qn, t0 + TPT) - 1;
+  const int kmin = max(0, ctx + t0 - window + 1);
+  const int32_t* bt = block_tables + (int64_t)s * bt_width;
+
+  // this lane's query slot as B fragments: [W_uk^T q (R) | rotated q (rd)], 8 dims at 32 kk + 8 g
+  xgk::bf16x8_t qf[NKK_MAX];
+  const int half = rot_dims >> 1;
+#pragma unroll
+  for (int kk = 0; kk < NKK_MAX; ++kk) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    const int d0 = kk * 32 + g * 8;
+    if (kk < nkk && valid && d0 < Dk) {
+      if (d0 < R) {
+        v = xgk::ld16(qabs + ((int64_t)head * Ttot + q0 + tok) * R + d0);
+      } else {
+        const int i0 = d0 - R;
+        const bf16* src = q + ((int64_t)(q0 + tok) * H + head) * dq + dn + i0;
+        float f[8];
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          const float a = bf2f(src[e]), b = bf2f(src[e + 1]);
+          if (i0 + e < rot_dims) {
+            const int pi = (i0 + e) >> 1;
+            const float c = rot[((int64_t)pos_q * half + pi) * 2], sn = rot[((int64_t)pos_q * half + pi) * 2 + 1];
+            f[e] = a * c - b * sn;
+            f[e + 1] = b * c + a * sn;
+          } else {
+            f[e] = a;
+            f[e + 1] = b;
+          }
+        }
+        v = xgk::pack8(f);
+      }
+    }
+    qf[kk] = xgk::as_frag(v);
+  }
+
+  xgk::f32x4_t o[NMT_MAX];
+#pragma unroll
+  for (int mt = 0; mt < NMT_MAX; ++mt) o[mt] = xgk::f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int cpk = nkk * 4;  // 16-byte chunks per staged row (zero padded to 32 nkk dims)
+  for (int k0 = kmin; k0 <= pos_last; k0 += kKT) {
+    __syncthreads();
+    for (int c = threadIdx.x; c < kKT * cpk; c += 256) {
+      const int key = c / cpk, ch = c - key * cpk;
+      const int kabs = k0 + key;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (kabs <= pos_last && ch * 8 < Dk)
+        v = xgk::ld16(cache + ((int64_t)bt[kabs / bs] * bs + kabs % bs) * Dk + ch * 8);
+      xgk::st16(tile_lds + key * LDK + ch * 8, v);
+    }
+    __syncthreads();
+    if (!wave_on) continue;
+    xgk::f32x4_t sacc[4];
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      sacc[n] = xgk::f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < NKK_MAX; ++kk)
+        if (kk < nkk)
+          sacc[n] = xgk::mfma16x16x32(xgk::as_frag(xgk::ld16(tile_lds + (n * 16 + li) * LDK + kk * 32 + g * 8)), qf[kk],
+                                      sacc[n]);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int kabs = k0 + n * 16 + g * 4 + r;
+        float v = sacc[n][r] * scale;
+        if (!valid || kabs > pos_q || kabs <= pos_q - window) v = -INFINITY;
+        sacc[n][r] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = m_new == -INFINITY ? 1.f : __expf(m - m_new);
+    float rs = 0.f;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = m_new == -INFINITY ? 0.f : __expf(sacc[n][r] - m_new);
+        sacc[n][r] = p;
+        rs += p;
+      }
+    rs += __shfl_xor(rs, 16, 64);
+    rs += __shfl_xor(rs, 32, 64);
+    l = l * alpha + rs;
+    m = m_new;
+#pragma unroll
+    for (int mt = 0; mt < NMT_MAX; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[mt][r] *= alpha;
+    // O^T += V^T . P^T over two 32-key chunks (keys in the order the score accumulator holds them)
+#pragma unroll
+    for (int sc = 0; sc < 2; ++sc) {
+      uint4 pb;
+      pb.x = xgk::pack2(sacc[2 * sc][0], sacc[2 * sc][1]);
+      pb.y = xgk::pack2(sacc[2 * sc][2], sacc[2 * sc][3]);
+      pb.z = xgk::pack2(sacc[2 * sc + 1][0], sacc[2 * sc + 1][1]);
+      pb.w = xgk::pack2(sacc[2 * sc + 1][2], sacc[2 * sc + 1][3]);
+      const xgk::bf16x8_t pfrag = xgk::as_frag(pb);
+      const int qq = li >> 2, pp = li & 3;
+      const int r0 = sc * 32 + 4 * g + qq, r1 = r0 + 16;
+#pragma unroll
+      for (int mt = 0; mt < NMT_MAX; ++mt)
+        if (mt < nmt) {
+          const xgk::bf16x4_t a0 = xgk::lds_read_tr16(tile_lds + r0 * LDK + mt * 16 + 4 * pp);
+          const xgk::bf16x4_t a1 = xgk::lds_read_tr16(tile_lds + r1 * LDK + mt * 16 + 4 * pp);
+          const xgk::bf16x8_t vfrag = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+          o[mt] = xgk::mfma16x16x32(vfrag, pfrag, o[mt]);
+        }
+    }
+  }
+  if (valid) {
+    const float gl = sigmoidf(bf2f(gate[(int64_t)(q0 + tok) * gate_stride + head])) * (l > 0.f ? 1.f / l : 0.f);
+    bf16* op = out + ((int64_t)head * Ttot + q0 + tok) * R;
+#pragma unroll
+    for (int mt = 0; mt < NMT_MAX; ++mt)
+      if (mt < nmt) {
+        uint2 w;
+        w.x = xgk::pack2(o[mt][0] * gl, o[mt][1] * gl);
+        w.y = xgk::pack2(o[mt][2] * gl, o[mt][3] * gl);
+        *reinterpret_cast<uint2*>(op + mt * 16 + 4 * g) = w;
+      }
+  }
+}
+
 // ------------------------------------------------------------------ generalized delta rule
 // One workgroup = (head, sequence); thread (col, ks) owns rows ks, ks + 4, .. of column col
 // of the [D x D] state, so u^T S and S^T r reduce over 4 neighbouring lanes only.
@@ -384,6 +546,101 @@ __global__ void delta_scan_kernel(const T* __restrict__ proj, int64_t ld, int of
       const int i = ks + kKS * r;
       if (i < D) st[(int64_t)i * D + col] = S[r];
     }
+  }
+}
+
+// ---- two-pass form: everything that does not depend on the state (decay, removal rate,
+// unit key) is computed once per (token, head) by a parallel kernel; the sequential scan
+// is then FMAs only, reads its per-token rows as 16-byte loads one token ahead, and each
+// thread owns RPT = D / 4 CONSECUTIVE rows of its column.
+// prep[t][h][5][D] fp32 = (w, a * u, u, k, r)
+template <typename T>
+__global__ void delta_prep_kernel(const T* __restrict__ proj, int64_t ld, int off_r, int off_k, int off_a,
+                                  const T* __restrict__ wl, int64_t ld_wl, const float* __restrict__ a_bias,
+                                  const float* __restrict__ w0, float* __restrict__ prep, int H, int D) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const T* row = proj + (int64_t)t * ld + h * D;
+  const T* wrow = wl + (int64_t)t * ld_wl + h * D;
+  float ksq = 0.f;
+  for (int d = lane; d < D; d += 64) {
+    const float k = ldf(row + off_k + d);
+    ksq += k * k;
+  }
+  ksq = wave_sum(ksq);
+  const float inv = 1.f / sqrtf(ksq + 1e-6f);
+  float* dst = prep + ((int64_t)t * H + h) * 5 * D;
+  for (int d = lane; d < D; d += 64) {
+    const float k = ldf(row + off_k + d), u = k * inv;
+    const float w = expf(-0.6065306597126334f * sigmoidf(ldf(wrow + d) + w0[h * D + d]));
+    const float a = sigmoidf(ldf(row + off_a + d) + a_bias[h * D + d]);
+    dst[d] = w;
+    dst[D + d] = a * u;
+    dst[2 * D + d] = u;
+    dst[3 * D + d] = k;
+    dst[4 * D + d] = ldf(row + off_r + d);
+  }
+}
+
+template <typename T, int RPT>
+__global__ __launch_bounds__(16 * RPT) void delta_scan2_kernel(const float* __restrict__ prep, const T* __restrict__ proj, int64_t ld, int off_v,
+                                   float* __restrict__ state, const int32_t* __restrict__ qsl,
+                                   const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots,
+                                   float* __restrict__ o, int H, int D) {
+  const int h = blockIdx.x, s = blockIdx.y;
+  const int q0 = qsl[s], q = qsl[s + 1] - q0, slot = slots[s];
+  if (slot < 0 || q <= 0) return;
+  const int ctx = seq_lens[s] - q;
+  const int col = threadIdx.x / kKS, ks = threadIdx.x % kKS;
+  const bool live = col < D;
+  const int cc = live ? col : 0;
+  const int r0 = ks * RPT;  // D == kKS * RPT
+  float S[RPT];
+  float* st = state + ((int64_t)slot * H + h) * D * D;
+#pragma unroll
+  for (int r = 0; r < RPT; ++r) S[r] = ctx > 0 ? st[(int64_t)(r0 + r) * D + cc] : 0.f;
+  constexpr int NV = RPT / 4;
+  float4 cur[5][NV], nxt[5][NV];
+  float vcur, vnxt = 0.f;
+  auto fetch = [&](int t, float4 (&dst)[5][NV], float& v) {
+    const float* src = prep + ((int64_t)(q0 + t) * H + h) * 5 * D + r0;
+#pragma unroll
+    for (int a = 0; a < 5; ++a)
+#pragma unroll
+      for (int i = 0; i < NV; ++i) dst[a][i] = *reinterpret_cast<const float4*>(src + a * D + 4 * i);
+    v = ldf(proj + (int64_t)(q0 + t) * ld + off_v + h * D + cc);
+  };
+  fetch(0, cur, vcur);
+  const int HD = H * D;
+  for (int t = 0; t < q; ++t) {
+    if (t + 1 < q) fetch(t + 1, nxt, vnxt);
+    const float* w = reinterpret_cast<const float*>(cur[0]);
+    const float* au = reinterpret_cast<const float*>(cur[1]);
+    const float* u = reinterpret_cast<const float*>(cur[2]);
+    const float* k = reinterpret_cast<const float*>(cur[3]);
+    const float* rr = reinterpret_cast<const float*>(cur[4]);
+    float uS = 0.f;
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) uS += u[r] * S[r];
+    uS += __shfl_xor(uS, 1, 64);
+    uS += __shfl_xor(uS, 2, 64);
+    float ot = 0.f;
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) {
+      S[r] = w[r] * S[r] - au[r] * uS + k[r] * vcur;
+      ot += S[r] * rr[r];
+    }
+    ot += __shfl_xor(ot, 1, 64);
+    ot += __shfl_xor(ot, 2, 64);
+    if (live && ks == 0) o[(int64_t)(q0 + t) * HD + h * D + col] = ot;
+#pragma unroll
+    for (int a = 0; a < 5; ++a)
+#pragma unroll
+      for (int i = 0; i < NV; ++i) cur[a][i] = nxt[a][i];
+    vcur = vnxt;
+  }
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) st[(int64_t)(r0 + r) * D + col] = S[r];
   }
 }
 
@@ -525,13 +782,68 @@ int latent_attention(const void* qabs, const void* q, bool f32, int64_t q_stride
   return -3;
 }
 
+template <int NMT_MAX>
+static int launch_latent_mfma(const void* qabs, const void* q, int dq, int dn, const void* gate, int64_t gate_stride,
+                              const void* cache, const int32_t* bt, int bt_width, int bs, const int32_t* qsl,
+                              const int32_t* seq_lens, const int32_t* slots, const float* rot, int rot_dims, void* out,
+                              int Ttot, int ns, int max_q, int H, int R, int rd, int window, float scale,
+                              hipStream_t st) {
+  const int nkk = (R + rd + 31) / 32;
+  const size_t bytes = (size_t)kKT * (nkk * 32 + 8) * sizeof(uint16_t);
+  auto kern = latent_attention_mfma_kernel<NMT_MAX>;
+  if (bytes > 48 * 1024) {
+    static bool set = false;
+    if (!set) {
+      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
+        return -2;
+      set = true;
+    }
+  }
+  const int TPT = max_q == 1 ? 1 : 16, HPT = max_q == 1 ? std::min(16, H) : 1;
+  dim3 grid((max_q + TPT - 1) / TPT, ns, (H + 4 * HPT - 1) / (4 * HPT));
+  kern<<<grid, 256, bytes, st>>>((const bf16*)qabs, (const bf16*)q, dq, dn, (const bf16*)gate, gate_stride,
+                                 (const bf16*)cache, bt, bt_width, bs, qsl, seq_lens, slots, rot, rot_dims, (bf16*)out,
+                                 Ttot, H, R, rd, window, scale, TPT, HPT);
+  return 0;
+}
+
+// bf16 only; R % 16 == 0, R <= 512, rd % 8 == 0, rd <= 128 (checked by the caller)
+int latent_attention_mfma(const void* qabs, const void* q, int dq, int dn, const void* gate, int64_t gate_stride,
+                          const void* cache, const int32_t* bt, int bt_width, int bs, const int32_t* qsl,
+                          const int32_t* seq_lens, const int32_t* slots, const float* rot, int rot_dims, void* out,
+                          int Ttot, int ns, int max_q, int H, int R, int rd, int window, float scale, hipStream_t st) {
+  if (Ttot <= 0 || ns <= 0 || max_q <= 0) return 0;
+  if (R % 16 || rd % 8 || R > 512 || rd > 128 || R < 16) return -1;
+#define XGM_LM(N)                                                                                                     \
+  return launch_latent_mfma<N>(qabs, q, dq, dn, gate, gate_stride, cache, bt, bt_width, bs, qsl, seq_lens, slots, rot, \
+                               rot_dims, out, Ttot, ns, max_q, H, R, rd, window, scale, st);
+  if (R <= 128) { XGM_LM(8) }
+  if (R <= 256) { XGM_LM(16) }
+  XGM_LM(32)
+#undef XGM_LM
+}
+
+// prep: fp32 scratch of Ttot * H * 5 * D floats, or null for the one-pass kernel
 int delta_scan(const void* proj, bool f32, int64_t ld, int off_r, int off_k, int off_v, int off_a, const void* wl,
                int64_t ld_wl, const float* a_bias, const float* w0, float* state, const int32_t* qsl,
-               const int32_t* seq_lens, const int32_t* slots, float* o, int ns, int H, int D, hipStream_t st) {
+               const int32_t* seq_lens, const int32_t* slots, float* o, int ns, int H, int D, float* prep, int Ttot,
+               hipStream_t st) {
   if (ns <= 0) return 0;
   const int threads = ((kKS * D + 63) / 64) * 64;
   if (threads > 1024) return -1;
   dim3 grid(H, ns);
+  if (prep != nullptr && (D == 16 || D == 32 || D == 64)) {
+    XGM_DISPATCH_T(f32, delta_prep_kernel<T><<<dim3(Ttot, H), 64, 0, st>>>((const T*)proj, ld, off_r, off_k, off_a,
+                                                                           (const T*)wl, ld_wl, a_bias, w0, prep, H, D);)
+#define XGM_DS2(RPT)                                                                                               \
+  XGM_DISPATCH_T(f32, delta_scan2_kernel<T, RPT><<<grid, threads, 0, st>>>(prep, (const T*)proj, ld, off_v, state, \
+                                                                            qsl, seq_lens, slots, o, H, D);)       \
+  return 0;
+    if (D == 16) { XGM_DS2(4) }
+    if (D == 32) { XGM_DS2(8) }
+    if (D == 64) { XGM_DS2(16) }
+#undef XGM_DS2
+  }
 #define XGM_DS(MAXR)                                                                                                  \
   XGM_DISPATCH_T(f32, delta_scan_kernel<T, MAXR><<<grid, threads, 0, st>>>((const T*)proj, ld, off_r, off_k, off_v,  \
                                                                             off_a, (const T*)wl, ld_wl, a_bias, w0,   \

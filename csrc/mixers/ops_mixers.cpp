@@ -20,8 +20,11 @@ void latent_prep(const void*, bool, int64_t, int, int, int, int, int, const floa
 int latent_attention(const void*, const void*, bool, int64_t, int, int, const void*, int64_t, const void*, const int32_t*,
                      int, int, const int32_t*, const int32_t*, const float*, int, void*, int, int, int, int, int, float,
                      hipStream_t);
+int latent_attention_mfma(const void*, const void*, int, int, const void*, int64_t, const void*, const int32_t*, int, int,
+                          const int32_t*, const int32_t*, const int32_t*, const float*, int, void*, int, int, int, int, int,
+                          int, int, float, hipStream_t);
 int delta_scan(const void*, bool, int64_t, int, int, int, int, const void*, int64_t, const float*, const float*, float*,
-               const int32_t*, const int32_t*, const int32_t*, float*, int, int, int, hipStream_t);
+               const int32_t*, const int32_t*, const int32_t*, float*, int, int, int, float*, int, hipStream_t);
 void delta_out(const float*, const float*, const void*, bool, int64_t, float, void*, int, int, int, hipStream_t);
 void xielu(const void*, bool, const float*, float, float, void*, int64_t, int, hipStream_t);
 void tanh_cols(const void*, bool, int64_t, void*, int, int, hipStream_t);
@@ -77,12 +80,25 @@ PYBIND11_MODULE(_mixers, m) {
                                    P<void>(out), T, H, R, rd, window, scale, S(st));
     check(rc, "latent_attention");
   });
+  m.def("latent_attention_mfma", [](uintptr_t qabs, uintptr_t q, int dq, int dn, uintptr_t gate, int64_t gate_stride,
+                                    uintptr_t cache, uintptr_t bt, int bt_width, int bs, uintptr_t qsl, uintptr_t sl,
+                                    uintptr_t slots, uintptr_t rot, int rot_dims, uintptr_t out, int T, int ns, int max_q,
+                                    int H, int R, int rd, int window, float scale, uintptr_t st) {
+    if (rot_dims % 2 || rot_dims > rd || dn + rd != dq || window < 1 || bs < 1)
+      throw std::invalid_argument("latent_attention_mfma: inconsistent sizes");
+    int rc = xgm::latent_attention_mfma(P<const void>(qabs), P<const void>(q), dq, dn, P<const void>(gate), gate_stride,
+                                        P<const void>(cache), P<const int32_t>(bt), bt_width, bs, P<const int32_t>(qsl),
+                                        P<const int32_t>(sl), P<const int32_t>(slots), P<const float>(rot), rot_dims,
+                                        P<void>(out), T, ns, max_q, H, R, rd, window, scale, S(st));
+    check(rc, "latent_attention_mfma");
+  });
   m.def("delta_scan", [](uintptr_t proj, bool f32, int64_t ld, int off_r, int off_k, int off_v, int off_a, uintptr_t wl,
                          int64_t ld_wl, uintptr_t a_bias, uintptr_t w0, uintptr_t state, uintptr_t qsl, uintptr_t sl,
-                         uintptr_t slots, uintptr_t o, int ns, int H, int D, uintptr_t st) {
+                         uintptr_t slots, uintptr_t o, int ns, int H, int D, uintptr_t prep, int T, uintptr_t st) {
     int rc = xgm::delta_scan(P<const void>(proj), f32, ld, off_r, off_k, off_v, off_a, P<const void>(wl), ld_wl,
                              P<const float>(a_bias), P<const float>(w0), P<float>(state), P<const int32_t>(qsl),
-                             P<const int32_t>(sl), P<const int32_t>(slots), P<float>(o), ns, H, D, S(st));
+                             P<const int32_t>(sl), P<const int32_t>(slots), P<float>(o), ns, H, D, P<float>(prep), T,
+                             S(st));
     check(rc, "delta_scan");
   });
   m.def("delta_out", [](uintptr_t o, uintptr_t nw, uintptr_t gate, bool f32, int64_t gate_stride, float eps, uintptr_t out,

@@ -18,6 +18,7 @@ from typing import Optional
 
 import torch
 
+from .. import tune
 from ._native import is_f32, mixers, native_device, stream_ptr
 
 
@@ -145,6 +146,10 @@ def _rotate_pairs(v: torch.Tensor, rot: torch.Tensor, pos: torch.Tensor, dims: i
 
 
 # ---------------------------------------------------------------------------- latent attention
+# XGS_TUNE latent_mfma=0: the general (any size, fp32-capable) kernel for bf16 too (A/B and tests)
+LATENT_MFMA = tune.get_bool("latent_mfma", True)
+
+
 def latent_prep(proj: torch.Tensor, off_q: int, Rq: int, off_kv: int, R: int, rd: int, wq: torch.Tensor,
                 wkv: Optional[torch.Tensor], eps: float, rot: torch.Tensor, rot_dims: int, sm: SeqMeta,
                 cache: Optional[torch.Tensor]) -> torch.Tensor:
@@ -190,6 +195,14 @@ def latent_attention(qabs: torch.Tensor, q: torch.Tensor, dn: int, gate: torch.T
         assert qabs.is_contiguous() and q.is_contiguous() and cache.is_contiguous() and gate.stride(1) == 1
         assert cache.dtype == qabs.dtype == q.dtype == gate.dtype and cache.shape[-1] == R + rd
         bt = _i32(sm.block_tables)
+        if LATENT_MFMA and qabs.dtype == torch.bfloat16 and R % 16 == 0 and 16 <= R <= 512 and rd % 8 == 0 and rd <= 128:
+            # matrix-core form: 16 query slots per wave, 64 cached rows per LDS tile
+            mixers().latent_attention_mfma(qabs.data_ptr(), q.data_ptr(), dq, dn, gate.data_ptr(), gate.stride(0),
+                                           cache.data_ptr(), bt.data_ptr(), bt.shape[1], block_size,
+                                           _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
+                                           _i32(sm.slots).data_ptr(), rot.data_ptr(), rot_dims, out.data_ptr(), T,
+                                           sm.num_seqs, sm.max_q, H, R, rd, int(window), float(scale), stream_ptr())
+            return out
         mixers().latent_attention(qabs.data_ptr(), q.data_ptr(), is_f32(q), H * dq, dq, dn, gate.data_ptr(),
                                   gate.stride(0), cache.data_ptr(), bt.data_ptr(), bt.shape[1], block_size,
                                   _i32(sm.positions).data_ptr(), _i32(sm.token_seq).data_ptr(), rot.data_ptr(), rot_dims,
@@ -226,6 +239,8 @@ def heads_to_rows(x: torch.Tensor) -> torch.Tensor:
 
 # ---------------------------------------------------------------------------- generalized delta rule
 DECAY_SCALE = math.exp(-0.5)
+# XGS_TUNE delta_two_pass=0: the one-pass scan kernel (any head size; A/B and tests)
+DELTA_TWO_PASS = tune.get_bool("delta_two_pass", True)
 UNIT_KEY_EPS = 1e-6
 
 
@@ -241,10 +256,12 @@ def delta_rule_scan(proj: torch.Tensor, off_r: int, off_k: int, off_v: int, off_
     if native_device(proj):
         assert proj.stride(1) == 1 and wl.stride(1) == 1 and wl.dtype == proj.dtype
         assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, D, D)
+        # state-independent terms (decay, removal rate, unit key) in a parallel pass of their own
+        prep = torch.empty(T * H * 5 * D, dtype=torch.float32, device=proj.device) if DELTA_TWO_PASS else None
         mixers().delta_scan(proj.data_ptr(), is_f32(proj), proj.stride(0), off_r, off_k, off_v, off_a, wl.data_ptr(),
                             wl.stride(0), a_bias.data_ptr(), w0.data_ptr(), state.data_ptr(), _i32(sm.qsl).data_ptr(),
                             _i32(sm.seq_lens).data_ptr(), _i32(sm.slots).data_ptr(), o.data_ptr(), sm.num_seqs, H, D,
-                            stream_ptr())
+                            _p(prep), T, stream_ptr())
         return o
     pf = proj.float()
     HD = H * D
