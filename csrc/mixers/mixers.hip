@@ -38,6 +38,23 @@ template <> __device__ __forceinline__ void stf<bf16>(bf16* p, float v) { *p = f
 
 __device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + expf(-x)); }
 
+// 4 consecutive elements (16-byte / 8-byte aligned)
+__device__ __forceinline__ void ld4(const float* p, float (&f)[4]) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x, f[1] = v.y, f[2] = v.z, f[3] = v.w;
+}
+__device__ __forceinline__ void ld4(const bf16* p, float (&f)[4]) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  f[0] = __uint_as_float(v.x << 16), f[1] = __uint_as_float(v.x & 0xFFFF0000u);
+  f[2] = __uint_as_float(v.y << 16), f[3] = __uint_as_float(v.y & 0xFFFF0000u);
+}
+__device__ __forceinline__ void st4(float* p, const float (&f)[4]) {
+  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+}
+__device__ __forceinline__ void st4(bf16* p, const float (&f)[4]) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(xgk::pack2(f[0], f[1]), xgk::pack2(f[2], f[3]));
+}
+
 // ------------------------------------------------------------------ embedding
 template <typename TW>
 __global__ void embed_rows_kernel(const int32_t* __restrict__ ids, const TW* __restrict__ table, float* __restrict__ out,
@@ -157,6 +174,48 @@ __global__ __launch_bounds__(256) void scaled_add_rmsnorm_kernel(const float* x,
     const float o = v * r * (w_offset + w[c]);
     if (x_out) x_out[(int64_t)t * W + c] = o;
     if (out) stf(out + (int64_t)t * W + c, o);
+  }
+}
+
+// one pass, 4 elements per access: W % 4 == 0, W <= 1024 NV, y rows 8-byte aligned
+template <typename TY, typename TO, int NV>
+__global__ __launch_bounds__(256) void scaled_add_rmsnorm_vec_kernel(const float* x, const TY* __restrict__ y,
+                                                                     int64_t y_stride, const float* __restrict__ bias,
+                                                                     float alpha, const float* __restrict__ w,
+                                                                     float w_offset, float eps, float* x_out,
+                                                                     TO* __restrict__ out, int W) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  float v[NV][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = 4 * (threadIdx.x + 256 * j);
+    if (c < W) {
+      ld4(x + (int64_t)t * W + c, v[j]);
+      float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
+      if (y) ld4(y + (int64_t)t * y_stride + c, a);
+      if (bias) ld4(bias + c, b);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[j][e] = alpha * v[j][e] + a[e] + b[e];
+        ss += v[j][e] * v[j][e];
+      }
+    }
+  }
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = 4 * (threadIdx.x + 256 * j);
+    if (c < W) {
+      float g[4], res[4];
+      ld4(w + c, g);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) res[e] = v[j][e] * r * (w_offset + g[e]);
+      if (x_out) st4(x_out + (int64_t)t * W + c, res);
+      if (out) st4(out + (int64_t)t * W + c, res);
+    }
   }
 }
 
@@ -386,18 +445,34 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
 #pragma unroll
   for (int mt = 0; mt < NMT_MAX; ++mt) o[mt] = xgk::f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  const int cpk = nkk * 4;  // 16-byte chunks per staged row (zero padded to 32 nkk dims)
+  // staging: thread -> (row = tid / 4, quarter = tid % 4) takes the row's 16-byte chunks quarter, quarter + 4, ..
+  // (4 nkk chunks per row, zero padded to 32 nkk dims): one page lookup per thread and tile, all loads of a
+  // tile in flight together, and (PREFETCH) the next tile's loads issued before this tile's MFMAs
+  constexpr bool PREFETCH = NMT_MAX <= 16;
+  const int srow = threadIdx.x >> 2, squad = threadIdx.x & 3;
+  uint4 stage[NKK_MAX];
+  auto fetch = [&](int k0) {
+    const int kabs = k0 + srow;
+    const bool ok = kabs <= pos_last;
+    const bf16* src = ok ? cache + ((int64_t)bt[kabs / bs] * bs + kabs % bs) * Dk : cache;
+#pragma unroll
+    for (int it = 0; it < NKK_MAX; ++it) {
+      const int ch = squad + 4 * it;
+      stage[it] = (it < nkk && ok && ch * 8 < Dk) ? xgk::ld16(src + ch * 8) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int it = 0; it < NKK_MAX; ++it)
+      if (it < nkk) xgk::st16(tile_lds + srow * LDK + (squad + 4 * it) * 8, stage[it]);
+  };
+  if (PREFETCH) fetch(kmin);
   for (int k0 = kmin; k0 <= pos_last; k0 += kKT) {
     __syncthreads();
-    for (int c = threadIdx.x; c < kKT * cpk; c += 256) {
-      const int key = c / cpk, ch = c - key * cpk;
-      const int kabs = k0 + key;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (kabs <= pos_last && ch * 8 < Dk)
-        v = xgk::ld16(cache + ((int64_t)bt[kabs / bs] * bs + kabs % bs) * Dk + ch * 8);
-      xgk::st16(tile_lds + key * LDK + ch * 8, v);
-    }
+    if (!PREFETCH) fetch(k0);
+    commit();
     __syncthreads();
+    if (PREFETCH && k0 + kKT <= pos_last) fetch(k0 + kKT);
     if (!wave_on) continue;
     xgk::f32x4_t sacc[4];
 #pragma unroll
@@ -581,6 +656,13 @@ __global__ void delta_prep_kernel(const T* __restrict__ proj, int64_t ld, int of
   }
 }
 
+// sum over the 4 lanes of a quad by DPP lane permutes (no LDS crossbar on the recurrence's critical path)
+__device__ __forceinline__ float quad_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));  // lane ^ 1
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));  // lane ^ 2
+  return v;
+}
+
 template <typename T, int RPT>
 __global__ __launch_bounds__(16 * RPT) void delta_scan2_kernel(const float* __restrict__ prep, const T* __restrict__ proj, int64_t ld, int off_v,
                                    float* __restrict__ state, const int32_t* __restrict__ qsl,
@@ -609,34 +691,35 @@ __global__ __launch_bounds__(16 * RPT) void delta_scan2_kernel(const float* __re
       for (int i = 0; i < NV; ++i) dst[a][i] = *reinterpret_cast<const float4*>(src + a * D + 4 * i);
     v = ldf(proj + (int64_t)(q0 + t) * ld + off_v + h * D + cc);
   };
-  fetch(0, cur, vcur);
   const int HD = H * D;
-  for (int t = 0; t < q; ++t) {
-    if (t + 1 < q) fetch(t + 1, nxt, vnxt);
-    const float* w = reinterpret_cast<const float*>(cur[0]);
-    const float* au = reinterpret_cast<const float*>(cur[1]);
-    const float* u = reinterpret_cast<const float*>(cur[2]);
-    const float* k = reinterpret_cast<const float*>(cur[3]);
-    const float* rr = reinterpret_cast<const float*>(cur[4]);
-    float uS = 0.f;
+  auto step = [&](int t, const float4 (&in)[5][NV], float v) {
+    const float* w = reinterpret_cast<const float*>(in[0]);
+    const float* au = reinterpret_cast<const float*>(in[1]);
+    const float* u = reinterpret_cast<const float*>(in[2]);
+    const float* k = reinterpret_cast<const float*>(in[3]);
+    const float* rr = reinterpret_cast<const float*>(in[4]);
+    float p[4] = {0.f, 0.f, 0.f, 0.f};  // four chains instead of one of RPT dependent FMAs
 #pragma unroll
-    for (int r = 0; r < RPT; ++r) uS += u[r] * S[r];
-    uS += __shfl_xor(uS, 1, 64);
-    uS += __shfl_xor(uS, 2, 64);
-    float ot = 0.f;
+    for (int r = 0; r < RPT; ++r) p[r & 3] += u[r] * S[r];
+    const float uS = quad_sum((p[0] + p[1]) + (p[2] + p[3]));
+    float c[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int r = 0; r < RPT; ++r) {
-      S[r] = w[r] * S[r] - au[r] * uS + k[r] * vcur;
-      ot += S[r] * rr[r];
+      S[r] = w[r] * S[r] - au[r] * uS + k[r] * v;
+      c[r & 3] += S[r] * rr[r];
     }
-    ot += __shfl_xor(ot, 1, 64);
-    ot += __shfl_xor(ot, 2, 64);
+    const float ot = quad_sum((c[0] + c[1]) + (c[2] + c[3]));
     if (live && ks == 0) o[(int64_t)(q0 + t) * HD + h * D + col] = ot;
-#pragma unroll
-    for (int a = 0; a < 5; ++a)
-#pragma unroll
-      for (int i = 0; i < NV; ++i) cur[a][i] = nxt[a][i];
-    vcur = vnxt;
+  };
+  // two register sets in turn: the rows of token t + 1 load while token t is computed
+  fetch(0, cur, vcur);
+  for (int t = 0; t < q; t += 2) {
+    if (t + 1 < q) fetch(t + 1, nxt, vnxt);
+    step(t, cur, vcur);
+    if (t + 1 < q) {
+      if (t + 2 < q) fetch(t + 2, cur, vcur);
+      step(t + 1, nxt, vnxt);
+    }
   }
   if (live) {
 #pragma unroll
@@ -669,6 +752,23 @@ __global__ void xielu_kernel(const T* __restrict__ in, const float* __restrict__
     if (bias) z += bias[i % F];
     const float y = z > 0.f ? sp * z * z + 0.5f * z : cn * (expm1f(z) - z) + 0.5f * z;
     stf(out + i, y);
+  }
+}
+
+// F % 4 == 0: 4 elements per access
+template <typename T>
+__global__ void xielu_vec_kernel(const T* __restrict__ in, const float* __restrict__ bias, float sp, float cn,
+                                 T* __restrict__ out, int64_t n4, int F) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+    float z[4], b[4] = {0.f, 0.f, 0.f, 0.f}, y[4];
+    ld4(in + 4 * i, z);
+    if (bias) ld4(bias + (4 * i) % F, b);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float v = z[e] + b[e];
+      y[e] = v > 0.f ? sp * v * v + 0.5f * v : cn * (expm1f(v) - v) + 0.5f * v;
+    }
+    st4(out + 4 * i, y);
   }
 }
 
@@ -719,12 +819,24 @@ void scaled_add_rmsnorm(const float* x, const void* y, bool y_f32, int64_t y_str
                         const float* w, float w_offset, float eps, float* x_out, void* out, bool out_f32, int T_, int W,
                         hipStream_t st) {
   if (T_ <= 0) return;
-#define XGM_SAR(TY, TO) \
-  scaled_add_rmsnorm_kernel<TY, TO><<<T_, 256, 0, st>>>(x, (const TY*)y, y_stride, bias, alpha, w, w_offset, eps, x_out, (TO*)out, W)
+  const int ysz = y_f32 ? 4 : 2;
+  const bool vec = W % 4 == 0 && W <= 8192 && (y == nullptr || ((uintptr_t)y % 16 == 0 && (y_stride * ysz) % 16 == 0));
+#define XGM_SAR(TY, TO)                                                                                                  \
+  {                                                                                                                      \
+    if (vec && W <= 2048)                                                                                                \
+      scaled_add_rmsnorm_vec_kernel<TY, TO, 2><<<T_, 256, 0, st>>>(x, (const TY*)y, y_stride, bias, alpha, w, w_offset, \
+                                                                    eps, x_out, (TO*)out, W);                            \
+    else if (vec)                                                                                                        \
+      scaled_add_rmsnorm_vec_kernel<TY, TO, 8><<<T_, 256, 0, st>>>(x, (const TY*)y, y_stride, bias, alpha, w, w_offset, \
+                                                                    eps, x_out, (TO*)out, W);                            \
+    else                                                                                                                 \
+      scaled_add_rmsnorm_kernel<TY, TO><<<T_, 256, 0, st>>>(x, (const TY*)y, y_stride, bias, alpha, w, w_offset, eps,    \
+                                                            x_out, (TO*)out, W);                                         \
+  }
   if (y_f32) {
-    if (out_f32) XGM_SAR(float, float); else XGM_SAR(float, bf16);
+    if (out_f32) XGM_SAR(float, float) else XGM_SAR(float, bf16)
   } else {
-    if (out_f32) XGM_SAR(bf16, float); else XGM_SAR(bf16, bf16);
+    if (out_f32) XGM_SAR(bf16, float) else XGM_SAR(bf16, bf16)
   }
 #undef XGM_SAR
 }
@@ -865,6 +977,11 @@ void delta_out(const float* o, const float* nw, const void* gate, bool f32, int6
 
 void xielu(const void* in, bool f32, const float* bias, float sp, float cn, void* out, int64_t n, int F, hipStream_t st) {
   if (n <= 0) return;
+  if (F % 4 == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    const int blocks4 = (int)std::min<int64_t>((n / 4 + 255) / 256, 1 << 20);
+    XGM_DISPATCH_T(f32, xielu_vec_kernel<T><<<blocks4, 256, 0, st>>>((const T*)in, bias, sp, cn, (T*)out, n / 4, F);)
+    return;
+  }
   const int blocks = (int)std::min<int64_t>((n + 255) / 256, 65535);
   XGM_DISPATCH_T(f32, xielu_kernel<T><<<blocks, 256, 0, st>>>((const T*)in, bias, sp, cn, (T*)out, n, F);)
 }
