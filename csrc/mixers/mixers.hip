@@ -381,7 +381,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
 // the B operand of O^T += V^T . P^T; V^T fragments are transposed LDS reads of the same tile.
 constexpr int kKT = 64;
 
-template <int NMT_MAX>
+template <int NMT_MAX, bool PREFETCH>
 __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const bf16* __restrict__ qabs, const bf16* __restrict__ q, int dq, int dn, const bf16* __restrict__ gate,
     int64_t gate_stride, const bf16* __restrict__ cache, const int32_t* __restrict__ block_tables, int bt_width, int bs,
@@ -447,8 +447,9 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   float m = -INFINITY, l = 0.f;
   // staging: thread -> (row = tid / 4, quarter = tid % 4) takes the row's 16-byte chunks quarter, quarter + 4, ..
   // (4 nkk chunks per row, zero padded to 32 nkk dims): one page lookup per thread and tile, all loads of a
-  // tile in flight together, and (PREFETCH) the next tile's loads issued before this tile's MFMAs
-  constexpr bool PREFETCH = NMT_MAX <= 16;
+  // tile in flight together, and (PREFETCH: single-token steps, whose few workgroups cannot hide the latency
+  // behind each other; it costs registers, so prompt portions rely on occupancy instead) the next tile's
+  // loads issued before this tile's MFMAs
   const int srow = threadIdx.x >> 2, squad = threadIdx.x & 3;
   uint4 stage[NKK_MAX];
   auto fetch = [&](int k0) {
@@ -664,67 +665,92 @@ __device__ __forceinline__ float quad_sum(float v) {
 }
 
 template <typename T, int RPT>
-__global__ __launch_bounds__(16 * RPT) void delta_scan2_kernel(const float* __restrict__ prep, const T* __restrict__ proj, int64_t ld, int off_v,
-                                   float* __restrict__ state, const int32_t* __restrict__ qsl,
-                                   const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots,
-                                   float* __restrict__ o, int H, int D) {
+__global__ __launch_bounds__(16 * RPT) void delta_scan2_kernel(const float* __restrict__ prep, const T* __restrict__ proj,
+                                                               int64_t ld, int off_v, float* __restrict__ state,
+                                                               const int32_t* __restrict__ qsl,
+                                                               const int32_t* __restrict__ seq_lens,
+                                                               const int32_t* __restrict__ slots, float* __restrict__ o,
+                                                               int H) {
+  constexpr int D = kKS * RPT, NT = kKS * D, CT = 16, ROW4 = 5 * D / 4, NV = RPT / 4;
+  // the per-token rows of CT tokens at a time, through LDS in two buffers: the next chunk's global
+  // loads are in flight while this chunk's CT sequential steps run
+  __shared__ float4 rows[2][CT][ROW4];
+  __shared__ float vals[2][CT][D];
   const int h = blockIdx.x, s = blockIdx.y;
   const int q0 = qsl[s], q = qsl[s + 1] - q0, slot = slots[s];
   if (slot < 0 || q <= 0) return;
   const int ctx = seq_lens[s] - q;
-  const int col = threadIdx.x / kKS, ks = threadIdx.x % kKS;
-  const bool live = col < D;
-  const int cc = live ? col : 0;
-  const int r0 = ks * RPT;  // D == kKS * RPT
+  const int tid = threadIdx.x, col = tid / kKS, ks = tid % kKS;
+  const int r0 = ks * RPT;
   float S[RPT];
   float* st = state + ((int64_t)slot * H + h) * D * D;
 #pragma unroll
-  for (int r = 0; r < RPT; ++r) S[r] = ctx > 0 ? st[(int64_t)(r0 + r) * D + cc] : 0.f;
-  constexpr int NV = RPT / 4;
-  float4 cur[5][NV], nxt[5][NV];
-  float vcur, vnxt = 0.f;
-  auto fetch = [&](int t, float4 (&dst)[5][NV], float& v) {
-    const float* src = prep + ((int64_t)(q0 + t) * H + h) * 5 * D + r0;
+  for (int r = 0; r < RPT; ++r) S[r] = ctx > 0 ? st[(int64_t)(r0 + r) * D + col] : 0.f;
+  float4 g[5];
+  float gv[4];
+  auto load_chunk = [&](int c) {
 #pragma unroll
-    for (int a = 0; a < 5; ++a)
-#pragma unroll
-      for (int i = 0; i < NV; ++i) dst[a][i] = *reinterpret_cast<const float4*>(src + a * D + 4 * i);
-    v = ldf(proj + (int64_t)(q0 + t) * ld + off_v + h * D + cc);
-  };
-  const int HD = H * D;
-  auto step = [&](int t, const float4 (&in)[5][NV], float v) {
-    const float* w = reinterpret_cast<const float*>(in[0]);
-    const float* au = reinterpret_cast<const float*>(in[1]);
-    const float* u = reinterpret_cast<const float*>(in[2]);
-    const float* k = reinterpret_cast<const float*>(in[3]);
-    const float* rr = reinterpret_cast<const float*>(in[4]);
-    float p[4] = {0.f, 0.f, 0.f, 0.f};  // four chains instead of one of RPT dependent FMAs
-#pragma unroll
-    for (int r = 0; r < RPT; ++r) p[r & 3] += u[r] * S[r];
-    const float uS = quad_sum((p[0] + p[1]) + (p[2] + p[3]));
-    float c[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int r = 0; r < RPT; ++r) {
-      S[r] = w[r] * S[r] - au[r] * uS + k[r] * v;
-      c[r & 3] += S[r] * rr[r];
+    for (int j = 0; j < 5; ++j) {
+      const int idx = tid + NT * j, tt = idx / ROW4, off = idx - tt * ROW4, t = c * CT + tt;
+      g[j] = t < q ? *reinterpret_cast<const float4*>(prep + ((int64_t)(q0 + t) * H + h) * 5 * D + 4 * off)
+                   : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    const float ot = quad_sum((c[0] + c[1]) + (c[2] + c[3]));
-    if (live && ks == 0) o[(int64_t)(q0 + t) * HD + h * D + col] = ot;
-  };
-  // two register sets in turn: the rows of token t + 1 load while token t is computed
-  fetch(0, cur, vcur);
-  for (int t = 0; t < q; t += 2) {
-    if (t + 1 < q) fetch(t + 1, nxt, vnxt);
-    step(t, cur, vcur);
-    if (t + 1 < q) {
-      if (t + 2 < q) fetch(t + 2, cur, vcur);
-      step(t + 1, nxt, vnxt);
-    }
-  }
-  if (live) {
 #pragma unroll
-    for (int r = 0; r < RPT; ++r) st[(int64_t)(r0 + r) * D + col] = S[r];
+    for (int j = 0; j < 4; ++j) {
+      const int idx = tid + NT * j, tt = idx / D, cc = idx - tt * D, t = c * CT + tt;
+      gv[j] = t < q ? ldf(proj + (int64_t)(q0 + t) * ld + off_v + h * D + cc) : 0.f;
+    }
+  };
+  auto store_chunk = [&](int b) {
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+      const int idx = tid + NT * j, tt = idx / ROW4;
+      rows[b][tt][idx - tt * ROW4] = g[j];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int idx = tid + NT * j, tt = idx / D;
+      vals[b][tt][idx - tt * D] = gv[j];
+    }
+  };
+  const int HD = H * D, nchunks = (q + CT - 1) / CT;
+  load_chunk(0);
+  store_chunk(0);
+  __syncthreads();
+  for (int c = 0; c < nchunks; ++c) {
+    const int b = c & 1;
+    if (c + 1 < nchunks) load_chunk(c + 1);
+    const int n = min(CT, q - c * CT);
+    for (int tt = 0; tt < n; ++tt) {
+      float4 in[5][NV];
+#pragma unroll
+      for (int a = 0; a < 5; ++a)
+#pragma unroll
+        for (int i = 0; i < NV; ++i) in[a][i] = rows[b][tt][a * (D / 4) + r0 / 4 + i];
+      const float v = vals[b][tt][col];
+      const float* w = reinterpret_cast<const float*>(in[0]);
+      const float* au = reinterpret_cast<const float*>(in[1]);
+      const float* u = reinterpret_cast<const float*>(in[2]);
+      const float* k = reinterpret_cast<const float*>(in[3]);
+      const float* rr = reinterpret_cast<const float*>(in[4]);
+      float p[4] = {0.f, 0.f, 0.f, 0.f};  // four chains instead of one of RPT dependent FMAs
+#pragma unroll
+      for (int r = 0; r < RPT; ++r) p[r & 3] += u[r] * S[r];
+      const float uS = quad_sum((p[0] + p[1]) + (p[2] + p[3]));
+      float a4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int r = 0; r < RPT; ++r) {
+        S[r] = w[r] * S[r] - au[r] * uS + k[r] * v;
+        a4[r & 3] += S[r] * rr[r];
+      }
+      const float ot = quad_sum((a4[0] + a4[1]) + (a4[2] + a4[3]));
+      if (ks == 0) o[(int64_t)(q0 + c * CT + tt) * HD + h * D + col] = ot;
+    }
+    if (c + 1 < nchunks) store_chunk(b ^ 1);
+    __syncthreads();
   }
+#pragma unroll
+  for (int r = 0; r < RPT; ++r) st[(int64_t)(r0 + r) * D + col] = S[r];
 }
 
 template <typename T>
@@ -902,13 +928,14 @@ static int launch_latent_mfma(const void* qabs, const void* q, int dq, int dn, c
                               hipStream_t st) {
   const int nkk = (R + rd + 31) / 32;
   const size_t bytes = (size_t)kKT * (nkk * 32 + 8) * sizeof(uint16_t);
-  auto kern = latent_attention_mfma_kernel<NMT_MAX>;
+  const bool prefetch = max_q == 1 && NMT_MAX <= 16;
+  auto kern = prefetch ? latent_attention_mfma_kernel<NMT_MAX, (NMT_MAX <= 16)> : latent_attention_mfma_kernel<NMT_MAX, false>;
   if (bytes > 48 * 1024) {
-    static bool set = false;
-    if (!set) {
+    static bool set[2] = {false, false};
+    if (!set[prefetch]) {
       if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
         return -2;
-      set = true;
+      set[prefetch] = true;
     }
   }
   const int TPT = max_q == 1 ? 1 : 16, HPT = max_q == 1 ? std::min(16, H) : 1;
@@ -949,7 +976,7 @@ int delta_scan(const void* proj, bool f32, int64_t ld, int off_r, int off_k, int
                                                                            (const T*)wl, ld_wl, a_bias, w0, prep, H, D);)
 #define XGM_DS2(RPT)                                                                                               \
   XGM_DISPATCH_T(f32, delta_scan2_kernel<T, RPT><<<grid, threads, 0, st>>>(prep, (const T*)proj, ld, off_v, state, \
-                                                                            qsl, seq_lens, slots, o, H, D);)       \
+                                                                            qsl, seq_lens, slots, o, H);)          \
   return 0;
     if (D == 16) { XGM_DS2(4) }
     if (D == 32) { XGM_DS2(8) }
