@@ -387,14 +387,16 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     int64_t gate_stride, const bf16* __restrict__ cache, const int32_t* __restrict__ block_tables, int bt_width, int bs,
     const int32_t* __restrict__ qsl, const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots,
     const float* __restrict__ rot, int rot_dims, bf16* __restrict__ out, int Ttot, int H, int R, int rd, int window,
-    float scale, int TPT, int HPT) {
+    float scale, int TPT, int HPT, int nsplit, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int NKK_MAX = NMT_MAX / 2 + 4;
   extern __shared__ __attribute__((aligned(16))) uint16_t tile_lds[];
   const int Dk = R + rd, nkk = (Dk + 31) >> 5, nmt = R >> 4, LDK = nkk * 32 + 8;
   const int s = blockIdx.y;
   const int q0 = qsl[s], qn = qsl[s + 1] - q0;
   if (slots[s] < 0 || qn <= 0) return;
-  const int t0 = blockIdx.x * TPT;
+  // nsplit > 1 (single-token steps): blockIdx.x is a share of the window's key tiles, merged by
+  // latent_attention_combine_kernel; else it is the tile of TPT tokens
+  const int t0 = nsplit > 1 ? 0 : blockIdx.x * TPT;
   if (t0 >= qn) return;
   const int ctx = seq_lens[s] - qn;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -404,8 +406,13 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   const int tl = li / HPT, head = h0 + li % HPT, tok = t0 + tl;
   const bool valid = wave_on && tl < TPT && tok < qn && head < H;
   const int pos_q = ctx + tok;
-  const int pos_last = ctx + min(qn, t0 + TPT) - 1;
-  const int kmin = max(0, ctx + t0 - window + 1);
+  int pos_last = ctx + min(qn, t0 + TPT) - 1;
+  int kmin = max(0, ctx + t0 - window + 1);
+  if (nsplit > 1) {
+    const int tiles = (pos_last - kmin + kKT) / kKT, per = (tiles + nsplit - 1) / nsplit;
+    kmin += blockIdx.x * per * kKT;
+    pos_last = min(pos_last, kmin + per * kKT - 1);  // may leave this share empty
+  }
   const int32_t* bt = block_tables + (int64_t)s * bt_width;
 
   // this lane's query slot as B fragments: [W_uk^T q (R) | rotated q (rd)], 8 dims at 32 kk + 8 g
@@ -538,7 +545,17 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
         }
     }
   }
-  if (valid) {
+  if (valid && nsplit > 1) {  // unnormalised share: (m, l) and the weighted latent sum
+    const int64_t row = ((int64_t)blockIdx.x * H + head) * Ttot + q0 + tok;
+    if (g == 0) {
+      part_ml[2 * row] = m;
+      part_ml[2 * row + 1] = l;
+    }
+#pragma unroll
+    for (int mt = 0; mt < NMT_MAX; ++mt)
+      if (mt < nmt)
+        *reinterpret_cast<float4*>(part_o + row * R + mt * 16 + 4 * g) = make_float4(o[mt][0], o[mt][1], o[mt][2], o[mt][3]);
+  } else if (valid) {
     const float gl = sigmoidf(bf2f(gate[(int64_t)(q0 + tok) * gate_stride + head])) * (l > 0.f ? 1.f / l : 0.f);
     bf16* op = out + ((int64_t)head * Ttot + q0 + tok) * R;
 #pragma unroll
@@ -549,6 +566,33 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
         w.y = xgk::pack2(o[mt][2] * gl, o[mt][3] * gl);
         *reinterpret_cast<uint2*>(op + mt * 16 + 4 * g) = w;
       }
+  }
+}
+
+// merge the key shares of a single-token step: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s, gated
+__global__ void latent_attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                const bf16* __restrict__ gate, int64_t gate_stride,
+                                                const int32_t* __restrict__ slots, bf16* __restrict__ out, int Ttot, int H,
+                                                int R, int nsplit) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  if (slots[t] < 0) return;  // single-token steps: row t is sequence t
+  float M = -INFINITY;
+  for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, part_ml[2 * (((int64_t)sp * H + h) * Ttot + t)]);
+  float L = 0.f;
+  for (int sp = 0; sp < nsplit; ++sp) {
+    const int64_t row = ((int64_t)sp * H + h) * Ttot + t;
+    const float ms = part_ml[2 * row];
+    if (ms != -INFINITY) L += __expf(ms - M) * part_ml[2 * row + 1];
+  }
+  const float gl = sigmoidf(bf2f(gate[(int64_t)t * gate_stride + h])) * (L > 0.f ? 1.f / L : 0.f);
+  for (int d = threadIdx.x; d < R; d += blockDim.x) {
+    float acc = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) {
+      const int64_t row = ((int64_t)sp * H + h) * Ttot + t;
+      const float ms = part_ml[2 * row];
+      if (ms != -INFINITY) acc += __expf(ms - M) * part_o[row * R + d];
+    }
+    out[((int64_t)h * Ttot + t) * R + d] = f2bf(acc * gl);
   }
 }
 
@@ -924,8 +968,8 @@ template <int NMT_MAX>
 static int launch_latent_mfma(const void* qabs, const void* q, int dq, int dn, const void* gate, int64_t gate_stride,
                               const void* cache, const int32_t* bt, int bt_width, int bs, const int32_t* qsl,
                               const int32_t* seq_lens, const int32_t* slots, const float* rot, int rot_dims, void* out,
-                              int Ttot, int ns, int max_q, int H, int R, int rd, int window, float scale,
-                              hipStream_t st) {
+                              int Ttot, int ns, int max_q, int H, int R, int rd, int window, float scale, int nsplit,
+                              float* part_o, float* part_ml, hipStream_t st) {
   const int nkk = (R + rd + 31) / 32;
   const size_t bytes = (size_t)kKT * (nkk * 32 + 8) * sizeof(uint16_t);
   const bool prefetch = max_q == 1 && NMT_MAX <= 16;
@@ -939,10 +983,14 @@ static int launch_latent_mfma(const void* qabs, const void* q, int dq, int dn, c
     }
   }
   const int TPT = max_q == 1 ? 1 : 16, HPT = max_q == 1 ? std::min(16, H) : 1;
-  dim3 grid((max_q + TPT - 1) / TPT, ns, (H + 4 * HPT - 1) / (4 * HPT));
+  if (max_q != 1 || part_o == nullptr || part_ml == nullptr) nsplit = 1;
+  dim3 grid(nsplit > 1 ? nsplit : (max_q + TPT - 1) / TPT, ns, (H + 4 * HPT - 1) / (4 * HPT));
   kern<<<grid, 256, bytes, st>>>((const bf16*)qabs, (const bf16*)q, dq, dn, (const bf16*)gate, gate_stride,
                                  (const bf16*)cache, bt, bt_width, bs, qsl, seq_lens, slots, rot, rot_dims, (bf16*)out,
-                                 Ttot, H, R, rd, window, scale, TPT, HPT);
+                                 Ttot, H, R, rd, window, scale, TPT, HPT, nsplit, part_o, part_ml);
+  if (nsplit > 1)
+    latent_attention_combine_kernel<<<dim3(Ttot, H), 64, 0, st>>>(part_o, part_ml, (const bf16*)gate, gate_stride, slots,
+                                                                  (bf16*)out, Ttot, H, R, nsplit);
   return 0;
 }
 
@@ -950,12 +998,14 @@ static int launch_latent_mfma(const void* qabs, const void* q, int dq, int dn, c
 int latent_attention_mfma(const void* qabs, const void* q, int dq, int dn, const void* gate, int64_t gate_stride,
                           const void* cache, const int32_t* bt, int bt_width, int bs, const int32_t* qsl,
                           const int32_t* seq_lens, const int32_t* slots, const float* rot, int rot_dims, void* out,
-                          int Ttot, int ns, int max_q, int H, int R, int rd, int window, float scale, hipStream_t st) {
+                          int Ttot, int ns, int max_q, int H, int R, int rd, int window, float scale, int nsplit,
+                          float* part_o, float* part_ml, hipStream_t st) {
   if (Ttot <= 0 || ns <= 0 || max_q <= 0) return 0;
+  if (nsplit > 1 && Ttot != ns) return -4;  // key shares are for steps of one token per sequence
   if (R % 16 || rd % 8 || R > 512 || rd > 128 || R < 16) return -1;
 #define XGM_LM(N)                                                                                                     \
   return launch_latent_mfma<N>(qabs, q, dq, dn, gate, gate_stride, cache, bt, bt_width, bs, qsl, seq_lens, slots, rot, \
-                               rot_dims, out, Ttot, ns, max_q, H, R, rd, window, scale, st);
+                               rot_dims, out, Ttot, ns, max_q, H, R, rd, window, scale, nsplit, part_o, part_ml, st);
   if (R <= 128) { XGM_LM(8) }
   if (R <= 256) { XGM_LM(16) }
   XGM_LM(32)

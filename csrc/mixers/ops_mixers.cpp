@@ -22,7 +22,7 @@ int latent_attention(const void*, const void*, bool, int64_t, int, int, const vo
                      hipStream_t);
 int latent_attention_mfma(const void*, const void*, int, int, const void*, int64_t, const void*, const int32_t*, int, int,
                           const int32_t*, const int32_t*, const int32_t*, const float*, int, void*, int, int, int, int, int,
-                          int, int, float, hipStream_t);
+                          int, int, float, int, float*, float*, hipStream_t);
 int delta_scan(const void*, bool, int64_t, int, int, int, int, const void*, int64_t, const float*, const float*, float*,
                const int32_t*, const int32_t*, const int32_t*, float*, int, int, int, float*, int, hipStream_t);
 void delta_out(const float*, const float*, const void*, bool, int64_t, float, void*, int, int, int, hipStream_t);
@@ -83,13 +83,15 @@ PYBIND11_MODULE(_mixers, m) {
   m.def("latent_attention_mfma", [](uintptr_t qabs, uintptr_t q, int dq, int dn, uintptr_t gate, int64_t gate_stride,
                                     uintptr_t cache, uintptr_t bt, int bt_width, int bs, uintptr_t qsl, uintptr_t sl,
                                     uintptr_t slots, uintptr_t rot, int rot_dims, uintptr_t out, int T, int ns, int max_q,
-                                    int H, int R, int rd, int window, float scale, uintptr_t st) {
-    if (rot_dims % 2 || rot_dims > rd || dn + rd != dq || window < 1 || bs < 1)
+                                    int H, int R, int rd, int window, float scale, int nsplit, uintptr_t part_o,
+                                    uintptr_t part_ml, uintptr_t st) {
+    if (rot_dims % 2 || rot_dims > rd || dn + rd != dq || window < 1 || bs < 1 || nsplit < 1)
       throw std::invalid_argument("latent_attention_mfma: inconsistent sizes");
     int rc = xgm::latent_attention_mfma(P<const void>(qabs), P<const void>(q), dq, dn, P<const void>(gate), gate_stride,
                                         P<const void>(cache), P<const int32_t>(bt), bt_width, bs, P<const int32_t>(qsl),
                                         P<const int32_t>(sl), P<const int32_t>(slots), P<const float>(rot), rot_dims,
-                                        P<void>(out), T, ns, max_q, H, R, rd, window, scale, S(st));
+                                        P<void>(out), T, ns, max_q, H, R, rd, window, scale, nsplit, P<float>(part_o),
+                                        P<float>(part_ml), S(st));
     check(rc, "latent_attention_mfma");
   });
   m.def("delta_scan", [](uintptr_t proj, bool f32, int64_t ld, int off_r, int off_k, int off_v, int off_a, uintptr_t wl,

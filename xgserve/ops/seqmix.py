@@ -148,6 +148,8 @@ def _rotate_pairs(v: torch.Tensor, rot: torch.Tensor, pos: torch.Tensor, dims: i
 # ---------------------------------------------------------------------------- latent attention
 # XGS_TUNE latent_mfma=0: the general (any size, fp32-capable) kernel for bf16 too (A/B and tests)
 LATENT_MFMA = tune.get_bool("latent_mfma", True)
+LATENT_MAX_SPLITS = 16    # key shares per single-token row, at most
+LATENT_SPLIT_WGS = 1024   # ... while the launch stays under about this many workgroups
 
 
 def latent_prep(proj: torch.Tensor, off_q: int, Rq: int, off_kv: int, R: int, rd: int, wq: torch.Tensor,
@@ -196,12 +198,21 @@ def latent_attention(qabs: torch.Tensor, q: torch.Tensor, dn: int, gate: torch.T
         assert cache.dtype == qabs.dtype == q.dtype == gate.dtype and cache.shape[-1] == R + rd
         bt = _i32(sm.block_tables)
         if LATENT_MFMA and qabs.dtype == torch.bfloat16 and R % 16 == 0 and 16 <= R <= 512 and rd % 8 == 0 and rd <= 128:
-            # matrix-core form: 16 query slots per wave, 64 cached rows per LDS tile
+            # matrix-core form: 16 query slots per wave, 64 cached rows per LDS tile; a step of single tokens
+            # divides each window's key tiles over several workgroups (merged by a second launch)
+            nsplit, part_o, part_ml = 1, None, None
+            if sm.max_q == 1 and T == sm.num_seqs:
+                groups = T * ((H + 4 * min(16, H) - 1) // (4 * min(16, H)))
+                nsplit = max(1, min(LATENT_MAX_SPLITS, (window + 63) // 64, LATENT_SPLIT_WGS // max(1, groups)))
+                if nsplit > 1:
+                    part_o = torch.empty(nsplit * H * T * R, dtype=torch.float32, device=q.device)
+                    part_ml = torch.empty(nsplit * H * T * 2, dtype=torch.float32, device=q.device)
             mixers().latent_attention_mfma(qabs.data_ptr(), q.data_ptr(), dq, dn, gate.data_ptr(), gate.stride(0),
                                            cache.data_ptr(), bt.data_ptr(), bt.shape[1], block_size,
                                            _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
                                            _i32(sm.slots).data_ptr(), rot.data_ptr(), rot_dims, out.data_ptr(), T,
-                                           sm.num_seqs, sm.max_q, H, R, rd, int(window), float(scale), stream_ptr())
+                                           sm.num_seqs, sm.max_q, H, R, rd, int(window), float(scale), nsplit,
+                                           _p(part_o), _p(part_ml), stream_ptr())
             return out
         mixers().latent_attention(qabs.data_ptr(), q.data_ptr(), is_f32(q), H * dq, dq, dn, gate.data_ptr(),
                                   gate.stride(0), cache.data_ptr(), bt.data_ptr(), bt.shape[1], block_size,
