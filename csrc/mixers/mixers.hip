@@ -800,7 +800,8 @@ __global__ __launch_bounds__(16 * RPT) void delta_scan2_kernel(const float* __re
 template <typename T>
 __global__ void delta_out_kernel(const float* __restrict__ o, const float* __restrict__ nw, const T* __restrict__ gate,
                                  int64_t gate_stride, float eps, T* __restrict__ out, int H, int D) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int t = blockIdx.x, h = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;  // a wave per head
+  if (h >= H) return;
   const float* row = o + ((int64_t)t * H + h) * D;
   float ss = 0.f;
   for (int d = lane; d < D; d += 64) ss += row[d] * row[d];
@@ -1049,7 +1050,7 @@ int delta_scan(const void* proj, bool f32, int64_t ld, int off_r, int off_k, int
 void delta_out(const float* o, const float* nw, const void* gate, bool f32, int64_t gate_stride, float eps, void* out,
                int T_, int H, int D, hipStream_t st) {
   if (T_ <= 0) return;
-  XGM_DISPATCH_T(f32, delta_out_kernel<T><<<dim3(T_, H), 64, 0, st>>>(o, nw, (const T*)gate, gate_stride, eps, (T*)out, H, D);)
+  XGM_DISPATCH_T(f32, delta_out_kernel<T><<<dim3(T_, (H + 3) / 4), 256, 0, st>>>(o, nw, (const T*)gate, gate_stride, eps, (T*)out, H, D);)
 }
 
 void xielu(const void* in, bool f32, const float* bias, float sp, float cn, void* out, int64_t n, int F, hipStream_t st) {
