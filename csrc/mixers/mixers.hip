@@ -381,14 +381,15 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
 // the B operand of O^T += V^T . P^T; V^T fragments are transposed LDS reads of the same tile.
 constexpr int kKT = 64;
 
-template <int NMT_MAX, bool PREFETCH>
+template <int NMT_MAX, bool PREFETCH, bool SPLIT>
 __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const bf16* __restrict__ qabs, const bf16* __restrict__ q, int dq, int dn, const bf16* __restrict__ gate,
     int64_t gate_stride, const bf16* __restrict__ cache, const int32_t* __restrict__ block_tables, int bt_width, int bs,
     const int32_t* __restrict__ qsl, const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots,
     const float* __restrict__ rot, int rot_dims, bf16* __restrict__ out, int Ttot, int H, int R, int rd, int window,
-    float scale, int TPT, int HPT, int nsplit, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float scale, int TPT, int HPT, int nsplit_arg, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int NKK_MAX = NMT_MAX / 2 + 4;
+  const int nsplit = SPLIT ? nsplit_arg : 1;  // prompt portions compile the key shares out (registers -> occupancy)
   extern __shared__ __attribute__((aligned(16))) uint16_t tile_lds[];
   const int Dk = R + rd, nkk = (Dk + 31) >> 5, nmt = R >> 4, LDK = nkk * 32 + 8;
   const int s = blockIdx.y;
@@ -973,14 +974,14 @@ static int launch_latent_mfma(const void* qabs, const void* q, int dq, int dn, c
                               float* part_o, float* part_ml, hipStream_t st) {
   const int nkk = (R + rd + 31) / 32;
   const size_t bytes = (size_t)kKT * (nkk * 32 + 8) * sizeof(uint16_t);
-  const bool prefetch = max_q == 1 && NMT_MAX <= 16;
-  auto kern = prefetch ? latent_attention_mfma_kernel<NMT_MAX, (NMT_MAX <= 16)> : latent_attention_mfma_kernel<NMT_MAX, false>;
+  auto kern = max_q == 1 ? latent_attention_mfma_kernel<NMT_MAX, (NMT_MAX <= 16), true>
+                         : latent_attention_mfma_kernel<NMT_MAX, false, false>;
   if (bytes > 48 * 1024) {
     static bool set[2] = {false, false};
-    if (!set[prefetch]) {
+    if (!set[max_q == 1]) {
       if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
         return -2;
-      set[prefetch] = true;
+      set[max_q == 1] = true;
     }
   }
   const int TPT = max_q == 1 ? 1 : 16, HPT = max_q == 1 ? std::min(16, H) : 1;
