@@ -16,7 +16,7 @@ import numpy as np
 
 def dofivik_layers(n_layers, heads, dim, rot, vdim, R, Rq, window, ff, d_heads, d_dim):
     att = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "kv_rank": R, "q_rank": Rq,
-           "scale": (dim + rot) ** -0.5, "mask": {"size": window}, "rot": {"base": 1e6, "dims": rot}}
+           "scale": (dim + rot) ** -0.5, "mask": {"size": window}, "rot": {"base": 5e5, "dims": rot}}
     out = []
     for i in range(n_layers):
         if i % 2 == 0:

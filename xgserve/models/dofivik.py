@@ -180,7 +180,7 @@ class DofivikLayer(nn.Module):
         return x
 
 
-def _lowrank_of(spec: dict, default: int = 16) -> int:
+def _lowrank_of(spec: dict, default: int = 32) -> int:
     return int(spec["mixer"].get("decay_rank", default))
 
 
