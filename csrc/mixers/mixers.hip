@@ -324,7 +324,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
   const int32_t* bt = block_tables + (int64_t)s * bt_width;
   for (int k0 = j0; k0 <= pos; k0 += KT) {
     const int n = min(KT, pos - k0 + 1);
-    __syncthreads();  // the previous tile is consumed (and qs is written, first time round)
+    __syncthreads();  // the previous tile is consumed (and qs is written, on the first pass)
     for (int jj = wave; jj < n; jj += 4) {
       const int key = k0 + jj;
       const T* src = cache + ((int64_t)bt[key / bs] * bs + key % bs) * Dk;
