@@ -323,10 +323,11 @@ def test_conv_carries_inputs_across_portions(device, taps):
 
 
 @pytest.mark.parametrize("device", OP_CASES)
-def test_norm_after_scaled_sum(device):
+@pytest.mark.parametrize("W", [77, 96, 2304])
+def test_norm_after_scaled_sum(device, W):
     g = torch.Generator().manual_seed(0)
-    x, y = torch.randn(9, 77, generator=g), torch.randn(9, 77, generator=g)
-    b, w = torch.randn(77, generator=g), torch.randn(77, generator=g) * 0.2
+    x, y = torch.randn(9, W, generator=g), torch.randn(9, W, generator=g)
+    b, w = torch.randn(W, generator=g), torch.randn(W, generator=g) * 0.2
     ref = orc.unit_rms(1.9 * x.to(F64) + y.to(F64) + b.to(F64), 1e-5) * (1 + w.to(F64))
     xd = x.clone().to(device)
     out = sq.scaled_add_rmsnorm(xd, y.to(device), w.to(device), 1e-5, 1.9, b.to(device), 1.0)
@@ -359,7 +360,8 @@ def latent_reference(qabs, qrot, lat, key, gate, window, scale):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-@pytest.mark.parametrize("shape", [(3, 24, 8, 5), (5, 32, 8, 8), (20, 48, 16, 4)], ids=["odd", "r32", "h20"])
+@pytest.mark.parametrize("shape", [(3, 24, 8, 5), (5, 32, 8, 8), (20, 48, 16, 4), (2, 160, 24, 8), (2, 288, 8, 4)],
+                         ids=["odd", "r32", "h20", "r160", "r288"])
 @pytest.mark.parametrize("window,bs", [(7, 4), (64, 16), (300, 16), (1, 4)])
 def test_latent_attention_one_key_stands_out(device, dtype, shape, window, bs):
     """For every query the key exactly `reach` back gets a dominating score, with reach = window - 1 (the
@@ -413,7 +415,7 @@ def test_latent_attention_one_key_stands_out(device, dtype, shape, window, bs):
 
 
 @pytest.mark.parametrize("device", OP_CASES)
-@pytest.mark.parametrize("H,D", [(3, 24), (2, 32), (2, 64), (1, 16)])
+@pytest.mark.parametrize("H,D", [(3, 24), (2, 32), (2, 64), (1, 16), (1, 128), (1, 72)])
 def test_delta_rule_state_over_portions_and_slots(device, H, D):
     """Head sizes of the one-pass kernel (any size) and of the two-pass one (16 / 32 / 64)."""
     W, eps = 40, 1e-5
