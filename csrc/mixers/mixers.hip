@@ -381,8 +381,8 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
 // the B operand of O^T += V^T . P^T; V^T fragments are transposed LDS reads of the same tile.
 constexpr int kKT = 64;
 
-template <int NMT_MAX, bool PREFETCH, bool SPLIT>
-__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
+template <int NMT_MAX, bool PREFETCH, bool SPLIT, int WPE>
+__global__ __launch_bounds__(256, WPE) void latent_attention_mfma_kernel(
     const bf16* __restrict__ qabs, const bf16* __restrict__ q, int dq, int dn, const bf16* __restrict__ gate,
     int64_t gate_stride, const bf16* __restrict__ cache, const int32_t* __restrict__ block_tables, int bt_width, int bs,
     const int32_t* __restrict__ qsl, const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots,
@@ -586,14 +586,22 @@ __global__ void latent_attention_combine_kernel(const float* __restrict__ part_o
     if (ms != -INFINITY) L += __expf(ms - M) * part_ml[2 * row + 1];
   }
   const float gl = sigmoidf(bf2f(gate[(int64_t)t * gate_stride + h])) * (L > 0.f ? 1.f / L : 0.f);
-  for (int d = threadIdx.x; d < R; d += blockDim.x) {
-    float acc = 0.f;
+  for (int d = 4 * threadIdx.x; d < R; d += 4 * blockDim.x) {  // R % 16 == 0
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int sp = 0; sp < nsplit; ++sp) {
       const int64_t row = ((int64_t)sp * H + h) * Ttot + t;
       const float ms = part_ml[2 * row];
-      if (ms != -INFINITY) acc += __expf(ms - M) * part_o[row * R + d];
+      if (ms != -INFINITY) {
+        const float e = __expf(ms - M);
+        float v[4];
+        ld4(part_o + row * R + d, v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += e * v[i];
+      }
     }
-    out[((int64_t)h * Ttot + t) * R + d] = f2bf(acc * gl);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] *= gl;
+    st4(out + ((int64_t)h * Ttot + t) * R + d, acc);
   }
 }
 
@@ -974,8 +982,9 @@ static int launch_latent_mfma(const void* qabs, const void* q, int dq, int dn, c
                               float* part_o, float* part_ml, hipStream_t st) {
   const int nkk = (R + rd + 31) / 32;
   const size_t bytes = (size_t)kKT * (nkk * 32 + 8) * sizeof(uint16_t);
-  auto kern = max_q == 1 ? latent_attention_mfma_kernel<NMT_MAX, (NMT_MAX <= 16), true>
-                         : latent_attention_mfma_kernel<NMT_MAX, false, false>;
+  // single-token steps walk one or two tiles per key share: no register prefetch, two waves per SIMD instead
+  auto kern = max_q == 1 ? latent_attention_mfma_kernel<NMT_MAX, false, true, (NMT_MAX <= 16 ? 2 : 1)>
+                         : latent_attention_mfma_kernel<NMT_MAX, false, false, 1>;
   if (bytes > 48 * 1024) {
     static bool set[2] = {false, false};
     if (!set[max_q == 1]) {
