@@ -381,7 +381,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
 // the B operand of O^T += V^T . P^T; V^T fragments are transposed LDS reads of the same tile.
 constexpr int kKT = 64;
 
-template <int NMT_MAX, bool PREFETCH, bool SPLIT, int WPE>
+template <int NMT_MAX, bool SPLIT, int WPE>
 __global__ __launch_bounds__(256, WPE) void latent_attention_mfma_kernel(
     const bf16* __restrict__ qabs, const bf16* __restrict__ q, int dq, int dn, const bf16* __restrict__ gate,
     int64_t gate_stride, const bf16* __restrict__ cache, const int32_t* __restrict__ block_tables, int bt_width, int bs,
@@ -455,9 +455,8 @@ __global__ __launch_bounds__(256, WPE) void latent_attention_mfma_kernel(
   float m = -INFINITY, l = 0.f;
   // staging: thread -> (row = tid / 4, quarter = tid % 4) takes the row's 16-byte chunks quarter, quarter + 4, ..
   // (4 nkk chunks per row, zero padded to 32 nkk dims): one page lookup per thread and tile, all loads of a
-  // tile in flight together, and (PREFETCH: single-token steps, whose few workgroups cannot hide the latency
-  // behind each other; it costs registers, so prompt portions rely on occupancy instead) the next tile's
-  // loads issued before this tile's MFMAs
+  // tile in flight together; latency is hidden by the other workgroups of the SIMD (two waves per SIMD up to a
+  // latent size of 256), single-token steps get them from the key shares
   const int srow = threadIdx.x >> 2, squad = threadIdx.x & 3;
   uint4 stage[NKK_MAX];
   auto fetch = [&](int k0) {
@@ -475,13 +474,11 @@ __global__ __launch_bounds__(256, WPE) void latent_attention_mfma_kernel(
     for (int it = 0; it < NKK_MAX; ++it)
       if (it < nkk) xgk::st16(tile_lds + srow * LDK + (squad + 4 * it) * 8, stage[it]);
   };
-  if (PREFETCH) fetch(kmin);
   for (int k0 = kmin; k0 <= pos_last; k0 += kKT) {
     __syncthreads();
-    if (!PREFETCH) fetch(k0);
+    fetch(k0);
     commit();
     __syncthreads();
-    if (PREFETCH && k0 + kKT <= pos_last) fetch(k0 + kKT);
     if (!wave_on) continue;
     xgk::f32x4_t sacc[4];
 #pragma unroll
@@ -982,9 +979,9 @@ static int launch_latent_mfma(const void* qabs, const void* q, int dq, int dn, c
                               float* part_o, float* part_ml, hipStream_t st) {
   const int nkk = (R + rd + 31) / 32;
   const size_t bytes = (size_t)kKT * (nkk * 32 + 8) * sizeof(uint16_t);
-  // single-token steps walk one or two tiles per key share: no register prefetch, two waves per SIMD instead
-  auto kern = max_q == 1 ? latent_attention_mfma_kernel<NMT_MAX, false, true, (NMT_MAX <= 16 ? 2 : 1)>
-                         : latent_attention_mfma_kernel<NMT_MAX, false, false, 1>;
+  // single-token steps walk one or two tiles per key share, at two waves per SIMD where the registers allow
+  auto kern = max_q == 1 ? latent_attention_mfma_kernel<NMT_MAX, true, (NMT_MAX <= 16 ? 2 : 1)>
+                         : latent_attention_mfma_kernel<NMT_MAX, false, 1>;
   if (bytes > 48 * 1024) {
     static bool set[2] = {false, false};
     if (!set[max_q == 1]) {
