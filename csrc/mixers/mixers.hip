@@ -17,64 +17,42 @@
 //
 // Activations / caches are T = float or bf16 (raw uint16_t); everything the recurrences,
 // norms, softmax and rotations touch is fp32.
-#include "common.h"
+#include "mixers_common.h"
 
 #include <algorithm>
 
 namespace xgm {
-using xgk::bf2f;
-using xgk::block_sum;
-using xgk::f2bf;
-using xgk::wave_max;
-using xgk::wave_sum;
-typedef uint16_t bf16;
-
-template <typename T> __device__ __forceinline__ float ldf(const T* p);
-template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
-template <> __device__ __forceinline__ float ldf<bf16>(const bf16* p) { return bf2f(*p); }
-template <typename T> __device__ __forceinline__ void stf(T* p, float v);
-template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
-template <> __device__ __forceinline__ void stf<bf16>(bf16* p, float v) { *p = f2bf(v); }
-
-__device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + expf(-x)); }
-
-// 4 consecutive elements (16-byte / 8-byte aligned)
-__device__ __forceinline__ void ld4(const float* p, float (&f)[4]) {
-  const float4 v = *reinterpret_cast<const float4*>(p);
-  f[0] = v.x, f[1] = v.y, f[2] = v.z, f[3] = v.w;
-}
-__device__ __forceinline__ void ld4(const bf16* p, float (&f)[4]) {
-  const uint2 v = *reinterpret_cast<const uint2*>(p);
-  f[0] = __uint_as_float(v.x << 16), f[1] = __uint_as_float(v.x & 0xFFFF0000u);
-  f[2] = __uint_as_float(v.y << 16), f[3] = __uint_as_float(v.y & 0xFFFF0000u);
-}
-__device__ __forceinline__ void st4(float* p, const float (&f)[4]) {
-  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
-}
-__device__ __forceinline__ void st4(bf16* p, const float (&f)[4]) {
-  *reinterpret_cast<uint2*>(p) = make_uint2(xgk::pack2(f[0], f[1]), xgk::pack2(f[2], f[3]));
-}
 
 // ------------------------------------------------------------------ embedding
+// pos_table != nullptr: + pos_table[positions[t]] (a learned vector per position, rows outside the table add nothing)
 template <typename TW>
 __global__ void embed_rows_kernel(const int32_t* __restrict__ ids, const TW* __restrict__ table, float* __restrict__ out,
-                                  int W, int V) {
+                                  int W, int V, const TW* __restrict__ pos_table, const int32_t* __restrict__ positions,
+                                  int P) {
   const int t = blockIdx.x;
   const int id = ids[t];
   const bool ok = id >= 0 && id < V;
-  for (int c = threadIdx.x; c < W; c += blockDim.x)
-    out[(int64_t)t * W + c] = ok ? ldf(table + (int64_t)id * W + c) : 0.f;
+  const int p = pos_table ? positions[t] : -1;
+  const bool pk = p >= 0 && p < P;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = ok ? ldf(table + (int64_t)id * W + c) : 0.f;
+    if (pk) v += ldf(pos_table + (int64_t)p * W + c);
+    out[(int64_t)t * W + c] = v;
+  }
 }
 
 // ------------------------------------------------------------------ causal conv with carried inputs
 constexpr int kMaxTaps = 8;
 
-// state[slot][k][c], k in [0, taps-1): the input at position ctx - (taps-1) + k (zero before the start)
-template <typename TO>
-__global__ void canon_conv_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ state,
+// state[slot][k][c], k in [0, taps-1): the input at position ctx - (taps-1) + k (zero before the start).
+// x is row-strided (ld_in) and float or bf16; out_t = [x_t if residual] + bias + sum_j w[:, j] x_(t-taps+1+j),
+// through silu when `act`; the state keeps raw inputs in fp32.
+template <typename TI, typename TO>
+__global__ void canon_conv_kernel(const TI* __restrict__ x, int64_t ld_in, const float* __restrict__ w,
+                                  const float* __restrict__ bias, float* __restrict__ state,
                                   const int32_t* __restrict__ qsl, const int32_t* __restrict__ seq_lens,
                                   const int32_t* __restrict__ slots, TO* __restrict__ out, int W, int taps, int tile,
-                                  int write_state) {
+                                  int write_state, int residual, int act) {
   const int s = blockIdx.z;
   const int q0 = qsl[s], q = qsl[s + 1] - q0, slot = slots[s];
   if (slot < 0 || q <= 0) return;
@@ -88,24 +66,26 @@ __global__ void canon_conv_kernel(const float* __restrict__ x, const float* __re
   float hist[kMaxTaps - 1], wt[kMaxTaps];
 #pragma unroll
   for (int j = 0; j < kMaxTaps; ++j) wt[j] = j < taps ? w[(int64_t)c * taps + j] : 0.f;
+  const float b = bias ? bias[c] : 0.f;
   float* st = state + ((int64_t)slot * nh) * W + c;
 #pragma unroll
   for (int j = 0; j < kMaxTaps - 1; ++j) {
     float v = 0.f;
     if (j < nh) {
       const int li = t0 - nh + j;  // local index of the input this tap history starts with
-      if (li >= 0) v = x[(int64_t)(q0 + li) * W + c];
+      if (li >= 0) v = ldf(x + (int64_t)(q0 + li) * ld_in + c);
       else if (ctx + li >= 0) v = st[(int64_t)(nh + li) * W];
     }
     hist[j] = v;
   }
   for (int t = t0; t < t1; ++t) {
-    const float cur = x[(int64_t)(q0 + t) * W + c];
-    float acc = cur;
+    const float cur = ldf(x + (int64_t)(q0 + t) * ld_in + c);
+    float acc = (residual ? cur : 0.f) + b;
 #pragma unroll
     for (int j = 0; j < kMaxTaps - 1; ++j)
       if (j < nh) acc += wt[j] * hist[j];
     acc += wt[nh] * cur;
+    if (act) acc = siluf(acc);
     stf(out + (int64_t)(q0 + t) * W + c, acc);
 #pragma unroll
     for (int j = 0; j < kMaxTaps - 1; ++j) {  // shift; the newest input goes last
@@ -121,9 +101,10 @@ __global__ void canon_conv_kernel(const float* __restrict__ x, const float* __re
 }
 
 // the carried rows after a step whose sequences were convolved by several tiles
-__global__ void canon_state_kernel(const float* __restrict__ x, float* __restrict__ state, const int32_t* __restrict__ qsl,
-                                   const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots, int W,
-                                   int taps) {
+template <typename TI>
+__global__ void canon_state_kernel(const TI* __restrict__ x, int64_t ld_in, float* __restrict__ state,
+                                   const int32_t* __restrict__ qsl, const int32_t* __restrict__ seq_lens,
+                                   const int32_t* __restrict__ slots, int W, int taps) {
   const int s = blockIdx.y;
   const int q0 = qsl[s], q = qsl[s + 1] - q0, slot = slots[s];
   if (slot < 0 || q <= 0) return;
@@ -138,7 +119,7 @@ __global__ void canon_state_kernel(const float* __restrict__ x, float* __restric
     v[j] = 0.f;
     if (j < nh) {
       const int li = q - nh + j;
-      if (li >= 0) v[j] = x[(int64_t)(q0 + li) * W + c];
+      if (li >= 0) v[j] = ldf(x + (int64_t)(q0 + li) * ld_in + c);
       else if (ctx + li >= 0) v[j] = st[(int64_t)(nh + li) * W];
     }
   }
@@ -866,30 +847,39 @@ __global__ void heads_to_rows_kernel(const T* __restrict__ in, T* __restrict__ o
 }
 
 // ================================================================== host launchers
-#define XGM_DISPATCH_T(f32, ...)      \
-  if (f32) {                          \
-    using T = float;                  \
-    __VA_ARGS__                       \
-  } else {                            \
-    using T = bf16;                   \
-    __VA_ARGS__                       \
-  }
-
-void embed_rows(const int32_t* ids, const void* table, bool f32, float* out, int T_, int W, int V, hipStream_t st) {
+void embed_rows(const int32_t* ids, const void* table, bool f32, float* out, int T_, int W, int V, const void* pos_table,
+                const int32_t* positions, int P, hipStream_t st) {
   if (T_ <= 0) return;
-  XGM_DISPATCH_T(f32, embed_rows_kernel<T><<<T_, 256, 0, st>>>(ids, (const T*)table, out, W, V);)
+  XGM_DISPATCH_T(f32, embed_rows_kernel<T><<<T_, 256, 0, st>>>(ids, (const T*)table, out, W, V, (const T*)pos_table,
+                                                                positions, P);)
 }
 
-void canon_conv(const float* x, const float* w, float* state, const int32_t* qsl, const int32_t* seq_lens,
-                const int32_t* slots, void* out, bool out_f32, int ns, int max_q, int W, int taps, hipStream_t st) {
+void causal_conv(const void* x, bool in_f32, int64_t ld_in, const float* w, const float* bias, float* state,
+                 const int32_t* qsl, const int32_t* seq_lens, const int32_t* slots, void* out, bool out_f32, int ns,
+                 int max_q, int W, int taps, bool residual, bool act, hipStream_t st) {
   if (ns <= 0 || max_q <= 0) return;
   const int tile = 64;
   const int ntiles = (max_q + tile - 1) / tile;
   dim3 grid((W + 255) / 256, ntiles, ns);
   const int ws = ntiles == 1 ? 1 : 0;
-  XGM_DISPATCH_T(out_f32, canon_conv_kernel<T><<<grid, 256, 0, st>>>(x, w, state, qsl, seq_lens, slots, (T*)out, W, taps,
-                                                                      tile, ws);)
-  if (!ws) canon_state_kernel<<<dim3((W + 255) / 256, ns), 256, 0, st>>>(x, state, qsl, seq_lens, slots, W, taps);
+#define XGM_CC(TI, TO)                                                                                                 \
+  canon_conv_kernel<TI, TO><<<grid, 256, 0, st>>>((const TI*)x, ld_in, w, bias, state, qsl, seq_lens, slots, (TO*)out, \
+                                                  W, taps, tile, ws, residual ? 1 : 0, act ? 1 : 0);
+  if (in_f32) {
+    if (out_f32) { XGM_CC(float, float) } else { XGM_CC(float, bf16) }
+  } else {
+    if (out_f32) { XGM_CC(bf16, float) } else { XGM_CC(bf16, bf16) }
+  }
+#undef XGM_CC
+  if (!ws) {
+    XGM_DISPATCH_T(in_f32, canon_state_kernel<T><<<dim3((W + 255) / 256, ns), 256, 0, st>>>((const T*)x, ld_in, state, qsl,
+                                                                                           seq_lens, slots, W, taps);)
+  }
+}
+
+void canon_conv(const float* x, const float* w, float* state, const int32_t* qsl, const int32_t* seq_lens,
+                const int32_t* slots, void* out, bool out_f32, int ns, int max_q, int W, int taps, hipStream_t st) {
+  causal_conv(x, true, W, w, nullptr, state, qsl, seq_lens, slots, out, out_f32, ns, max_q, W, taps, true, false, st);
 }
 
 void scaled_add_rmsnorm(const float* x, const void* y, bool y_f32, int64_t y_stride, const float* bias, float alpha,

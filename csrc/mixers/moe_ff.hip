@@ -1,0 +1,339 @@
+// Gated feed-forward pieces and a routed mixture of small experts.
+//
+//   glu_act          [gate | up] rows -> act(gate) * up':
+//                      kGluGeluTanh   0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * u
+//                      kGluClamped    g' = min(g, limit), u' = clamp(u, -limit, limit):  g' sigmoid(alpha g') (u' + 1)
+//   grouped_router   fp32 router logits -> sigmoid scores; choice scores = score + correction; experts form
+//                    `count` equal groups of neighbours, a group scores the sum of its two largest choice
+//                    scores, only experts of the best `keep` groups can be chosen (the others count as
+//                    -inf); the `top` largest choice scores win; weights = score (WITHOUT correction) * scale
+//   moe_align        (token, choice) pairs sorted by expert into tiles of kTileM rows (padded with -1)
+//   grouped_gemm     per tile: rows x expert weights; first GEMM with the gated activation fused,
+//                    second GEMM to fp32 rows
+//   moe_combine      out[t] = sum_j weight[t, j] * y[row of pair (t, j)]   (fixed order: bit-stable)
+//
+// Activations / weights are T = float or bf16; router, weights of the sum and the sum itself are fp32.
+#include "mixers_common.h"
+
+#include <algorithm>
+
+namespace xgm {
+
+constexpr int kGluGeluTanh = 0, kGluClamped = 1;
+constexpr int kTileM = 16;  // rows per expert tile
+
+__device__ __forceinline__ float glu(int kind, float g, float u, float limit, float alpha) {
+  if (kind == kGluGeluTanh) {
+    const float c = 0.7978845608028654f;  // sqrt(2 / pi)
+    return 0.5f * g * (1.f + tanhf(c * (g + 0.044715f * g * g * g))) * u;
+  }
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g * sigmoidf(alpha * g) * (u + 1.f);
+}
+
+template <typename T>
+__global__ void glu_act_kernel(const T* __restrict__ in, int64_t ld, T* __restrict__ out, int F, int64_t total, int kind,
+                               float limit, float alpha) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = i / F;
+    const int c = (int)(i % F);
+    const T* row = in + t * ld;
+    stf(out + i, glu(kind, ldf(row + c), ldf(row + F + c), limit, alpha));
+  }
+}
+
+// ------------------------------------------------------------------ router: one wave per token
+constexpr int kMaxEPL = 8;  // experts per lane: E <= 512
+
+__global__ __launch_bounds__(64) void grouped_router_kernel(const float* __restrict__ logits, const float* __restrict__ corr,
+                                                            int E, int count, int keep, int top, float scale,
+                                                            int32_t* __restrict__ ids, float* __restrict__ wts) {
+  extern __shared__ float sm[];
+  float* cs = sm;              // [E] choice scores
+  float* gs = sm + E;          // [count] group scores
+  int* kept = (int*)(gs + count);  // [count]
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const int per = E / count;
+  float sc[kMaxEPL], ch[kMaxEPL];
+#pragma unroll
+  for (int i = 0; i < kMaxEPL; ++i) {
+    const int e = lane + 64 * i;
+    sc[i] = 0.f, ch[i] = -INFINITY;
+    if (e < E) {
+      sc[i] = sigmoidf(logits[(int64_t)t * E + e]);
+      ch[i] = sc[i] + (corr ? corr[e] : 0.f);
+      cs[e] = ch[i];
+    }
+  }
+  __syncthreads();
+  for (int g = lane; g < count; g += 64) {  // sum of the group's two largest choice scores
+    float a = -INFINITY, b = -INFINITY;
+    for (int j = 0; j < per; ++j) {
+      const float v = cs[g * per + j];
+      if (v > a) b = a, a = v;
+      else if (v > b) b = v;
+    }
+    gs[g] = per > 1 ? a + b : a;
+  }
+  __syncthreads();
+  for (int g = lane; g < count; g += 64) {  // rank among the groups (ties: the lower index first)
+    int rank = 0;
+    const float v = gs[g];
+    for (int o = 0; o < count; ++o) rank += (gs[o] > v || (gs[o] == v && o < g)) ? 1 : 0;
+    kept[g] = rank < keep ? 1 : 0;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kMaxEPL; ++i) {
+    const int e = lane + 64 * i;
+    if (e < E && !kept[e / per]) ch[i] = -INFINITY;
+  }
+  for (int j = 0; j < top; ++j) {
+    float bv = -INFINITY, bs = 0.f;
+    int be = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < kMaxEPL; ++i) {
+      const int e = lane + 64 * i;
+      if (e < E && (ch[i] > bv || (ch[i] == bv && e < be))) bv = ch[i], be = e, bs = sc[i];
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64), os = __shfl_xor(bs, o, 64);
+      const int oe = __shfl_xor(be, o, 64);
+      if (ov > bv || (ov == bv && oe < be)) bv = ov, be = oe, bs = os;
+    }
+    if (be >= E) be = 0, bs = 0.f;  // fewer candidates than `top`: expert 0 with weight 0
+    if (lane == 0) {
+      ids[(int64_t)t * top + j] = be;
+      wts[(int64_t)t * top + j] = bs * scale;
+    }
+#pragma unroll
+    for (int i = 0; i < kMaxEPL; ++i)
+      if (lane + 64 * i == be) ch[i] = -INFINITY;
+  }
+}
+
+// ------------------------------------------------------------------ pairs -> expert tiles (one workgroup)
+__global__ __launch_bounds__(1024) void moe_align_kernel(const int32_t* __restrict__ ids, int pairs, int E, int cap,
+                                                         int32_t* __restrict__ rows, int32_t* __restrict__ tile_expert,
+                                                         int32_t* __restrict__ dest) {
+  extern __shared__ int si[];
+  int* cnt = si;          // [E]
+  int* off = si + E;      // [E + 1] padded starts
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) atomicAdd(&cnt[ids[i]], 1);
+  for (int i = threadIdx.x; i < cap; i += blockDim.x) rows[i] = -1;
+  for (int i = threadIdx.x; i < cap / kTileM; i += blockDim.x) tile_expert[i] = -1;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int o = 0;
+    for (int e = 0; e < E; ++e) {
+      off[e] = o;
+      o += (cnt[e] + kTileM - 1) / kTileM * kTileM;
+    }
+    off[E] = o;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    for (int tl = off[e] / kTileM; tl < off[e + 1] / kTileM; ++tl) tile_expert[tl] = e;
+    cnt[e] = 0;  // becomes the fill cursor
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+    const int e = ids[i];
+    const int r = off[e] + atomicAdd(&cnt[e], 1);
+    rows[r] = i;
+    dest[i] = r;
+  }
+}
+
+// ------------------------------------------------------------------ grouped GEMM, general form
+// Tile = kTileM rows x 64 columns, 256 threads: thread (tr = tid / 16, tc = tid % 16) owns row tr and
+// columns tc + 16 j. K runs through LDS in chunks of 32. GATED: the weight holds [gate (F rows) | up (F rows)]
+// and the output column f is glu(gate_f, up_f); A rows are gathered through rows[] / top.
+template <typename T, bool GATED>
+__global__ __launch_bounds__(256) void grouped_gemm_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ Wt,
+                                                           const int32_t* __restrict__ rows,
+                                                           const int32_t* __restrict__ tile_expert, int top, int Nout,
+                                                           int K, void* __restrict__ out, int kind, float limit,
+                                                           float alpha) {
+  __shared__ float As[kTileM][33];
+  __shared__ float Ws[64][33];
+  __shared__ float Us[GATED ? 64 : 1][33];
+  const int tile = blockIdx.x;
+  const int e = tile_expert[tile];
+  if (e < 0) return;
+  const int n0 = blockIdx.y * 64;
+  const int tr = threadIdx.x >> 4, tc = threadIdx.x & 15;
+  const int r = tile * kTileM + tr;
+  const int pr = rows[r];
+  const int64_t wrows = GATED ? 2 * (int64_t)Nout : (int64_t)Nout;
+  const T* We = Wt + (int64_t)e * wrows * K;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f}, accu[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < kTileM * 32; i += 256) {
+      const int rr = i >> 5, kk = i & 31;
+      const int p2 = rows[tile * kTileM + rr];
+      float v = 0.f;
+      if (p2 >= 0 && k0 + kk < K) v = ldf(A + (int64_t)(GATED ? p2 / top : tile * kTileM + rr) * lda + k0 + kk);
+      As[rr][kk] = v;
+    }
+    for (int i = threadIdx.x; i < 64 * 32; i += 256) {
+      const int nn = i >> 5, kk = i & 31;
+      const bool ok = n0 + nn < Nout && k0 + kk < K;
+      Ws[nn][kk] = ok ? ldf(We + (int64_t)(n0 + nn) * K + k0 + kk) : 0.f;
+      if (GATED) Us[nn][kk] = ok ? ldf(We + (int64_t)(Nout + n0 + nn) * K + k0 + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < 32; ++kk) {
+      const float a = As[tr][kk];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[j] += a * Ws[tc + 16 * j][kk];
+        if (GATED) accu[j] += a * Us[tc + 16 * j][kk];
+      }
+    }
+  }
+  if (pr < 0) return;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + tc + 16 * j;
+    if (n >= Nout) continue;
+    if (GATED) stf((T*)out + (int64_t)r * Nout + n, glu(kind, acc[j], accu[j], limit, alpha));
+    else ((float*)out)[(int64_t)r * Nout + n] = acc[j];
+  }
+}
+
+// ---- matrix-core form (bf16; K % 32 == 0, Nout % 16 == 0): one wave = 16 rows x 16 NT columns,
+// A / B fragments straight from global memory (16 bytes per lane), fp32 accumulators.
+using xgk::as_frag;
+using xgk::f32x4_t;
+using xgk::ld16;
+using xgk::mfma16x16x32;
+
+template <bool GATED, int NT>
+__global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __restrict__ A, int64_t lda,
+                                                                const bf16* __restrict__ Wt,
+                                                                const int32_t* __restrict__ rows,
+                                                                const int32_t* __restrict__ tile_expert, int top,
+                                                                int Nout, int K, void* __restrict__ out, int kind,
+                                                                float limit, float alpha) {
+  const int tile = blockIdx.x;
+  const int e = tile_expert[tile];
+  if (e < 0) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = (blockIdx.y * 4 + wave) * 16 * NT;
+  if (n0 >= Nout) return;
+  const int l16 = lane & 15, kg = lane >> 4;
+  const int64_t wrows = GATED ? 2 * (int64_t)Nout : (int64_t)Nout;
+  const bf16* We = Wt + (int64_t)e * wrows * K;
+  const int pa = rows[tile * kTileM + l16];
+  const bf16* arow = A + (int64_t)(GATED ? max(pa, 0) / top : tile * kTileM + l16) * lda + kg * 8;
+  f32x4_t acc[NT], accu[GATED ? NT : 1];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < (GATED ? NT : 1); ++j) accu[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const uint4 av = pa >= 0 ? ld16(arow + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int n = n0 + 16 * j + l16;
+      if (n0 + 16 * j < Nout) {  // whole 16-column tiles only (Nout % 16 == 0)
+        // D = A(rows x k) B(k x cols): rows come out along the accumulator's 4 entries x (lane >> 4)
+        acc[j] = mfma16x16x32(as_frag(av), as_frag(ld16(We + (int64_t)n * K + k0 + kg * 8)), acc[j]);
+        if (GATED) accu[j] = mfma16x16x32(as_frag(av), as_frag(ld16(We + (int64_t)(Nout + n) * K + k0 + kg * 8)), accu[j]);
+      }
+    }
+  }
+  // accumulator entry i of lane (l16, kg): row kg * 4 + i, column l16
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int n = n0 + 16 * j + l16;
+    if (n0 + 16 * j >= Nout) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int rr = tile * kTileM + kg * 4 + i;
+      if (rows[rr] < 0) continue;
+      if (GATED) ((bf16*)out)[(int64_t)rr * Nout + n] = f2bf(glu(kind, acc[j][i], accu[j][i], limit, alpha));
+      else ((float*)out)[(int64_t)rr * Nout + n] = acc[j][i];
+    }
+  }
+}
+
+__global__ void moe_combine_kernel(const float* __restrict__ y, const int32_t* __restrict__ dest,
+                                   const float* __restrict__ wts, int top, int W, float* __restrict__ out) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < top; ++j) acc += wts[(int64_t)t * top + j] * y[(int64_t)dest[(int64_t)t * top + j] * W + c];
+    out[(int64_t)t * W + c] = acc;
+  }
+}
+
+// ================================================================== host launchers
+void glu_act(const void* in, bool f32, int64_t ld, void* out, int T_, int F, int kind, float limit, float alpha,
+             hipStream_t st) {
+  const int64_t total = (int64_t)T_ * F;
+  if (total <= 0) return;
+  const int blocks = (int)std::min<int64_t>((total + 255) / 256, 1 << 16);
+  XGM_DISPATCH_T(f32, glu_act_kernel<T><<<blocks, 256, 0, st>>>((const T*)in, ld, (T*)out, F, total, kind, limit, alpha);)
+}
+
+int grouped_router(const float* logits, const float* corr, int T_, int E, int count, int keep, int top, float scale,
+                   int32_t* ids, float* wts, hipStream_t st) {
+  if (T_ <= 0) return 0;
+  if (E < 1 || E > 64 * kMaxEPL || count < 1 || E % count != 0 || keep < 1 || keep > count || top < 1 ||
+      top > keep * (E / count))
+    return -1;
+  grouped_router_kernel<<<T_, 64, (E + 2 * count) * sizeof(float), st>>>(logits, corr, E, count, keep, top, scale, ids, wts);
+  return 0;
+}
+
+int moe_align(const int32_t* ids, int pairs, int E, int cap, int32_t* rows, int32_t* tile_expert, int32_t* dest,
+              hipStream_t st) {
+  if (pairs <= 0) return 0;
+  if (E < 1 || E > 4096 || cap % kTileM != 0 || cap < pairs + E * (kTileM - 1)) return -1;
+  moe_align_kernel<<<1, 1024, (2 * E + 1) * sizeof(int), st>>>(ids, pairs, E, cap, rows, tile_expert, dest);
+  return 0;
+}
+
+int grouped_gemm(const void* A, bool f32, int64_t lda, const void* Wt, const int32_t* rows, const int32_t* tile_expert,
+                 int cap, int top, int Nout, int K, bool gated, void* out, int kind, float limit, float alpha, bool mfma,
+                 hipStream_t st) {
+  if (cap <= 0) return 0;
+  if (cap % kTileM != 0 || Nout < 1 || K < 1) return -1;
+  const int tiles = cap / kTileM;
+  if (!f32 && mfma && K % 32 == 0 && Nout % 16 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)Wt % 16 == 0) {
+    constexpr int NT = 2;
+    dim3 grid(tiles, (Nout + 64 * NT - 1) / (64 * NT));
+    if (gated)
+      grouped_gemm_mfma_kernel<true, NT><<<grid, 256, 0, st>>>((const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top,
+                                                               Nout, K, out, kind, limit, alpha);
+    else
+      grouped_gemm_mfma_kernel<false, NT><<<grid, 256, 0, st>>>((const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert,
+                                                                top, Nout, K, out, kind, limit, alpha);
+    return 0;
+  }
+  dim3 grid(tiles, (Nout + 63) / 64);
+  if (gated) {
+    XGM_DISPATCH_T(f32, grouped_gemm_kernel<T, true><<<grid, 256, 0, st>>>((const T*)A, lda, (const T*)Wt, rows, tile_expert,
+                                                                            top, Nout, K, out, kind, limit, alpha);)
+  } else {
+    XGM_DISPATCH_T(f32, grouped_gemm_kernel<T, false><<<grid, 256, 0, st>>>((const T*)A, lda, (const T*)Wt, rows,
+                                                                             tile_expert, top, Nout, K, out, kind, limit,
+                                                                             alpha);)
+  }
+  return 0;
+}
+
+void moe_combine(const float* y, const int32_t* dest, const float* wts, int T_, int top, int W, float* out, hipStream_t st) {
+  if (T_ <= 0) return;
+  moe_combine_kernel<<<T_, 256, 0, st>>>(y, dest, wts, top, W, out);
+}
+
+}  // namespace xgm

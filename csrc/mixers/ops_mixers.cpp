@@ -10,7 +10,25 @@
 namespace py = pybind11;
 
 namespace xgm {
-void embed_rows(const int32_t*, const void*, bool, float*, int, int, int, hipStream_t);
+void embed_rows(const int32_t*, const void*, bool, float*, int, int, int, const void*, const int32_t*, int, hipStream_t);
+void causal_conv(const void*, bool, int64_t, const float*, const float*, float*, const int32_t*, const int32_t*,
+                 const int32_t*, void*, bool, int, int, int, int, bool, bool, hipStream_t);
+void residual_norm(float*, const void*, int64_t, const float*, const void*, int64_t, const float*, const float*, bool,
+                   const float*, float, float*, void*, bool, int, int, hipStream_t);
+void qk_norm_cache(const void*, bool, int64_t, int, int, int, const float*, const float*, float, const int32_t*, void*,
+                   void*, void*, int, hipStream_t);
+int masked_attention(const void*, bool, const void*, const void*, const int32_t*, int, int, const int32_t*,
+                     const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, float,
+                     hipStream_t);
+int ssm_scan(const void*, bool, int64_t, const void*, int64_t, const float*, const float*, const float*, float*,
+             const int32_t*, const int32_t*, const int32_t*, float*, int, int, int, int, int, hipStream_t);
+void gated_group_norm(const float*, const void*, bool, int64_t, const float*, float, void*, int, int, int, hipStream_t);
+void glu_act(const void*, bool, int64_t, void*, int, int, int, float, float, hipStream_t);
+int grouped_router(const float*, const float*, int, int, int, int, int, float, int32_t*, float*, hipStream_t);
+int moe_align(const int32_t*, int, int, int, int32_t*, int32_t*, int32_t*, hipStream_t);
+int grouped_gemm(const void*, bool, int64_t, const void*, const int32_t*, const int32_t*, int, int, int, int, bool, void*,
+                 int, float, float, bool, hipStream_t);
+void moe_combine(const float*, const int32_t*, const float*, int, int, int, float*, hipStream_t);
 void canon_conv(const float*, const float*, float*, const int32_t*, const int32_t*, const int32_t*, void*, bool, int, int,
                 int, int, hipStream_t);
 void scaled_add_rmsnorm(const float*, const void*, bool, int64_t, const float*, float, const float*, float, float, float*,
@@ -41,10 +59,98 @@ static void check(int rc, const char* what) {
 }
 
 PYBIND11_MODULE(_mixers, m) {
-  m.def("embed_rows", [](uintptr_t ids, uintptr_t table, bool f32, uintptr_t out, int T, int W, int V, uintptr_t st) {
-    xgm::embed_rows(P<const int32_t>(ids), P<const void>(table), f32, P<float>(out), T, W, V, S(st));
+  m.def("embed_rows", [](uintptr_t ids, uintptr_t table, bool f32, uintptr_t out, int T, int W, int V, uintptr_t pos_table,
+                         uintptr_t positions, int Pn, uintptr_t st) {
+    if (pos_table && !positions) throw std::invalid_argument("embed_rows: a position table needs positions");
+    xgm::embed_rows(P<const int32_t>(ids), P<const void>(table), f32, P<float>(out), T, W, V, P<const void>(pos_table),
+                    P<const int32_t>(positions), Pn, S(st));
     check(0, "embed_rows");
   });
+  m.def("causal_conv", [](uintptr_t x, bool in_f32, int64_t ld_in, uintptr_t w, uintptr_t bias, uintptr_t state,
+                          uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t out, bool out_f32, int ns, int max_q,
+                          int C, int taps, bool residual, bool act, uintptr_t st) {
+    if (taps < 1 || taps > 8) throw std::invalid_argument("causal_conv: taps must be in [1, 8]");
+    if (ld_in < C) throw std::invalid_argument("causal_conv: row stride smaller than the channel count");
+    xgm::causal_conv(P<const void>(x), in_f32, ld_in, P<const float>(w), P<const float>(bias), P<float>(state),
+                     P<const int32_t>(qsl), P<const int32_t>(sl), P<const int32_t>(slots), P<void>(out), out_f32, ns,
+                     max_q, C, taps, residual, act, S(st));
+    check(0, "causal_conv");
+  });
+  m.def("residual_norm", [](uintptr_t x, uintptr_t y1, int64_t ld1, uintptr_t a1, uintptr_t y2, int64_t ld2, uintptr_t y3,
+                            uintptr_t a2, bool y_f32, uintptr_t g, float eps, uintptr_t n32, uintptr_t nact,
+                            bool nact_f32, int T, int W, uintptr_t st) {
+    if ((y1 && ld1 < W) || (y2 && ld2 < W)) throw std::invalid_argument("residual_norm: row stride smaller than the width");
+    xgm::residual_norm(P<float>(x), P<const void>(y1), ld1, P<const float>(a1), P<const void>(y2), ld2, P<const float>(y3),
+                       P<const float>(a2), y_f32, P<const float>(g), eps, P<float>(n32), P<void>(nact), nact_f32, T, W,
+                       S(st));
+    check(0, "residual_norm");
+  });
+  m.def("qk_norm_cache", [](uintptr_t proj, bool f32, int64_t ld, int nq, int nk, int nv, uintptr_t wq, uintptr_t wk,
+                            float eps, uintptr_t slot_mapping, uintptr_t q_out, uintptr_t kcache, uintptr_t vcache, int T,
+                            uintptr_t st) {
+    if (nq < 1 || nk < 1 || nv < 1 || ld < nq + nk + nv) throw std::invalid_argument("qk_norm_cache: inconsistent sizes");
+    xgm::qk_norm_cache(P<const void>(proj), f32, ld, nq, nk, nv, P<const float>(wq), P<const float>(wk), eps,
+                       P<const int32_t>(slot_mapping), P<void>(q_out), P<void>(kcache), P<void>(vcache), T, S(st));
+    check(0, "qk_norm_cache");
+  });
+  m.def("masked_attention", [](uintptr_t q, bool f32, uintptr_t kc, uintptr_t vc, uintptr_t bt, int bt_width, int bs,
+                               uintptr_t pos, uintptr_t token_seq, uintptr_t temp, uintptr_t sink, uintptr_t out, int T,
+                               int H, int G, int dk, int dv, int mask, int size, float scale, uintptr_t st) {
+    if (bs < 1 || bt_width < 1) throw std::invalid_argument("masked_attention: inconsistent sizes");
+    int rc = xgm::masked_attention(P<const void>(q), f32, P<const void>(kc), P<const void>(vc), P<const int32_t>(bt),
+                                   bt_width, bs, P<const int32_t>(pos), P<const int32_t>(token_seq), P<const float>(temp),
+                                   P<const float>(sink), P<void>(out), T, H, G, dk, dv, mask, size, scale, S(st));
+    check(rc, "masked_attention");
+  });
+  m.def("ssm_scan", [](uintptr_t xbc, bool f32, int64_t ld_x, uintptr_t dt, int64_t ld_dt, uintptr_t dt_bias,
+                       uintptr_t A_log, uintptr_t D, uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots,
+                       uintptr_t y, int ns, int H, int G, int N, int Pd, uintptr_t st) {
+    if (H < 1 || G < 1 || ld_x < (int64_t)H * Pd + 2 * (int64_t)G * N || ld_dt < H)
+      throw std::invalid_argument("ssm_scan: inconsistent sizes");
+    int rc = xgm::ssm_scan(P<const void>(xbc), f32, ld_x, P<const void>(dt), ld_dt, P<const float>(dt_bias),
+                           P<const float>(A_log), P<const float>(D), P<float>(state), P<const int32_t>(qsl),
+                           P<const int32_t>(sl), P<const int32_t>(slots), P<float>(y), ns, H, G, N, Pd, S(st));
+    check(rc, "ssm_scan");
+  });
+  m.def("gated_group_norm", [](uintptr_t y, uintptr_t z, bool f32, int64_t ld_z, uintptr_t w, float eps, uintptr_t out,
+                               int T, int inner, int ng, uintptr_t st) {
+    if (ng < 1 || inner % ng) throw std::invalid_argument("gated_group_norm: the parts must divide the row");
+    xgm::gated_group_norm(P<const float>(y), P<const void>(z), f32, ld_z, P<const float>(w), eps, P<void>(out), T, inner,
+                          ng, S(st));
+    check(0, "gated_group_norm");
+  });
+  m.def("glu_act", [](uintptr_t in, bool f32, int64_t ld, uintptr_t out, int T, int F, int kind, float limit, float alpha,
+                      uintptr_t st) {
+    if (kind < 0 || kind > 1 || ld < 2 * (int64_t)F) throw std::invalid_argument("glu_act: inconsistent arguments");
+    xgm::glu_act(P<const void>(in), f32, ld, P<void>(out), T, F, kind, limit, alpha, S(st));
+    check(0, "glu_act");
+  });
+  m.def("grouped_router", [](uintptr_t logits, uintptr_t corr, int T, int E, int count, int keep, int top, float scale,
+                             uintptr_t ids, uintptr_t wts, uintptr_t st) {
+    int rc = xgm::grouped_router(P<const float>(logits), P<const float>(corr), T, E, count, keep, top, scale,
+                                 P<int32_t>(ids), P<float>(wts), S(st));
+    check(rc, "grouped_router");
+  });
+  m.def("moe_align", [](uintptr_t ids, int pairs, int E, int cap, uintptr_t rows, uintptr_t tile_expert, uintptr_t dest,
+                        uintptr_t st) {
+    int rc = xgm::moe_align(P<const int32_t>(ids), pairs, E, cap, P<int32_t>(rows), P<int32_t>(tile_expert),
+                            P<int32_t>(dest), S(st));
+    check(rc, "moe_align");
+  });
+  m.def("grouped_gemm", [](uintptr_t A, bool f32, int64_t lda, uintptr_t Wt, uintptr_t rows, uintptr_t tile_expert, int cap,
+                           int top, int Nout, int K, bool gated, uintptr_t out, int kind, float limit, float alpha,
+                           bool mfma, uintptr_t st) {
+    if (top < 1 || lda < K) throw std::invalid_argument("grouped_gemm: inconsistent sizes");
+    int rc = xgm::grouped_gemm(P<const void>(A), f32, lda, P<const void>(Wt), P<const int32_t>(rows),
+                               P<const int32_t>(tile_expert), cap, top, Nout, K, gated, P<void>(out), kind, limit, alpha,
+                               mfma, S(st));
+    check(rc, "grouped_gemm");
+  });
+  m.def("moe_combine", [](uintptr_t y, uintptr_t dest, uintptr_t wts, int T, int top, int W, uintptr_t out, uintptr_t st) {
+    xgm::moe_combine(P<const float>(y), P<const int32_t>(dest), P<const float>(wts), T, top, W, P<float>(out), S(st));
+    check(0, "moe_combine");
+  });
+  m.attr("MOE_TILE_M") = 16;
   m.def("canon_conv", [](uintptr_t x, uintptr_t w, uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots,
                          uintptr_t out, bool out_f32, int ns, int max_q, int W, int taps, uintptr_t st) {
     if (taps < 1 || taps > 8) throw std::invalid_argument("canon_conv: taps must be in [1, 8]");

@@ -135,7 +135,7 @@ def build_kernels(force: bool = False, jobs: int = 8, probes: bool = False) -> P
 def build_mixers(force: bool = False, jobs: int = 8) -> Path:
     srcs = sorted((CSRC / "mixers").glob("*.hip"))
     cpp = sorted((CSRC / "mixers").glob("*.cpp"))
-    hdrs = [CSRC / "kernels" / "common.h"]
+    hdrs = [CSRC / "kernels" / "common.h"] + sorted((CSRC / "mixers").glob("*.h"))
     out = PKG / f"_mixers{EXT}"
     flags = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-fvisibility=hidden", "-Wno-unused-result",
              *NO_PK_F32]
@@ -144,7 +144,7 @@ def build_mixers(force: bool = False, jobs: int = 8) -> Path:
         return out
     obj_dir = BUILD / "mixers"
     obj_dir.mkdir(parents=True, exist_ok=True)
-    inc = _pybind_includes() + [f"-I{CSRC / 'kernels'}"]
+    inc = _pybind_includes() + [f"-I{CSRC / 'kernels'}", f"-I{CSRC / 'mixers'}"]
 
     def cc(src):
         o = obj_dir / (src.stem + ".o")

@@ -16,7 +16,7 @@ from typing import Dict, List, Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                      # "llama" | "mixtral" | "gpt2" | "dofivik"
+    arch: str                      # "llama" | "mixtral" | "gpt2" | "dofivik" | "vizonex"
     hidden_size: int
     num_layers: int
     num_heads: int
@@ -34,7 +34,7 @@ class ModelConfig:
     bos_token_id: int = 1
     eos_token_ids: List[int] = field(default_factory=lambda: [2])
     dtype: str = "bfloat16"
-    # layer-list architectures ("dofivik"): one dict per layer {"type", "mixer", "mlp"}, the
+    # layer-list architectures ("dofivik", "vizonex"): one dict per layer {"type", "mixer", "mlp"}, the
     # residual scale of the norm-after-sum sublayers, and the taps of the input convolution
     layer_specs: Optional[List[dict]] = None
     postln_alpha: float = 1.0
@@ -51,7 +51,10 @@ class ModelConfig:
     def num_params(self) -> int:
         H, F, V, L = self.hidden_size, self.intermediate_size, self.vocab_size, self.num_layers
         if self.layer_specs is not None:
-            from .dofivik import count_params
+            if self.arch == "vizonex":
+                from .vizonex import count_params
+            else:
+                from .dofivik import count_params
             return count_params(self)
         attn = H * (self.q_size + 2 * self.kv_size) + self.q_size * H
         if self.arch == "mixtral":
@@ -64,6 +67,9 @@ class ModelConfig:
         return L * (attn + mlp + 2 * H) + emb + H
 
     def kv_bytes_per_token(self, tp: int = 1, dtype_bytes: int = 2) -> int:
+        if self.arch == "vizonex":
+            return sum((m["dim"] + m["vdim"]) * m["kv_heads"] * dtype_bytes
+                       for m in (L["mixer"] for L in self.layer_specs if L["type"] == "attention"))
         if self.layer_specs is not None:
             return sum((m["kv_rank"] + m["rot_dim"]) * dtype_bytes for m in (L["mixer"] for L in self.layer_specs)
                        if "kv_rank" in m and "kv_from" not in m)
@@ -141,6 +147,71 @@ def _dofivik_tiny_layers():
 
 
 register(dofivik_config("dofivik-tiny", 128, 512, _dofivik_tiny_layers(), max_position=1024))
+
+
+def vizonex_config(name: str, width: int, vocab: int, layers: List[dict], taps: int = 4, eps: float = 1e-6,
+                   max_position: int = 4096) -> ModelConfig:
+    """A Vizonex model: learned position vectors and a list of parallel blocks x + a1 mixer(n + conv(n)) + a2 ff(n),
+    n = rmsnorm(x). Mixers: "attention" (grouped-query, whole-vector q / k norms, chunked visibility, per-head
+    temperature and softmax sink) and "mamba2" (scalar-decay state-space recurrence). Feed-forward: "dense"
+    (gelu-tanh gate), "moe" (grouped sigmoid router over clamped-GLU experts + a shared expert) or none."""
+    def need(d, keys, where):
+        for k in keys:
+            if k not in d:
+                raise ValueError(f"{where}: missing {k!r}")
+    if taps < 1 or taps > 8:
+        raise ValueError("canon.taps must be in [1, 8]")
+    for i, L in enumerate(layers):
+        m, w = L.get("mixer") or {}, f"layer {i}"
+        if L.get("type") == "attention":
+            need(m, ("heads", "kv_heads", "dim", "vdim", "scale", "mask"), w)
+            if m["heads"] % m["kv_heads"] or int(m["mask"]["size"]) < 1:
+                raise ValueError(f"{w}: heads must be a multiple of kv_heads and mask.size positive")
+        elif L.get("type") == "mamba2":
+            need(m, ("heads", "vdim", "state", "groups", "norm_groups", "conv"), w)
+            if m["heads"] % m["groups"] or (m["heads"] * m["vdim"]) % m["norm_groups"] or not 1 <= m["conv"] <= 8:
+                raise ValueError(f"{w}: heads must be a multiple of groups, heads * vdim of norm_groups, conv in [1, 8]")
+            if m["state"] > 256:
+                raise ValueError(f"{w}: state sizes above 256 are not supported")
+        else:
+            raise ValueError(f"{w}: unknown mixer type {L.get('type')!r}")
+        mlp = L.get("mlp")
+        if mlp is None:
+            continue
+        if mlp.get("kind") == "dense":
+            need(mlp, ("ff",), w)
+        elif mlp.get("kind") == "moe":
+            need(mlp, ("expert", "router"), w)
+            r = mlp["router"]
+            need(r, ("experts", "top", "groups", "scale"), w)
+            E, c, k = r["experts"], r["groups"]["count"], r["groups"]["keep"]
+            if E % c or not 1 <= k <= c or not 1 <= r["top"] <= k * (E // c) or E > 512:
+                raise ValueError(f"{w}: experts must divide into groups.count groups, 1 <= keep <= count, "
+                                 "top <= keep * group size, experts <= 512")
+        else:
+            raise ValueError(f"{w}: unknown feed-forward kind {mlp.get('kind')!r}")
+    att = [L["mixer"] for L in layers if L["type"] == "attention"]
+    heads = max([L["mixer"]["heads"] for L in layers] or [1])
+    hd = max([max(m["dim"], m["vdim"]) for m in att] or [L["mixer"]["vdim"] for L in layers] or [1])
+    ffs = [(L["mlp"]["ff"] if L["mlp"]["kind"] == "dense" else
+            L["mlp"]["expert"]["ff"] * L["mlp"]["router"]["top"] + (L["mlp"].get("shared") or {}).get("ff", 0))
+           for L in layers if L.get("mlp")]
+    return ModelConfig(name, "vizonex", width, len(layers), heads, max([m["kv_heads"] for m in att] or [1]), hd,
+                       max(ffs or [0]), vocab, max_position, 0.0, None, eps, False, bos_token_id=0, eos_token_ids=[],
+                       layer_specs=layers, canon_taps=int(taps))
+
+
+def _vizonex_tiny_layers():
+    att = {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 16, "scale": 0.2, "mask": {"size": 24}}
+    ssm = {"heads": 4, "vdim": 16, "state": 16, "groups": 2, "norm_groups": 2, "conv": 3}
+    moe = {"kind": "moe", "expert": {"ff": 32, "limit": 3.0}, "shared": {"ff": 48, "limit": 2.0},
+           "router": {"experts": 8, "top": 2, "scale": 1.25, "groups": {"count": 4, "keep": 2}}}
+    return [{"type": "attention", "mixer": dict(att), "mlp": {"kind": "dense", "ff": 192}},
+            {"type": "mamba2", "mixer": dict(ssm), "mlp": moe},
+            {"type": "attention", "mixer": dict(att), "mlp": None}]
+
+
+register(vizonex_config("vizonex-tiny", 128, 512, _vizonex_tiny_layers(), taps=3, max_position=1024))
 register(ModelConfig("gpt2-tiny", "gpt2", 128, 2, 2, 2, 64, 512, 512, 256, 0.0, tie_embeddings=True,
                      bos_token_id=0, eos_token_ids=[0], dtype="float32"))
 
@@ -163,6 +234,9 @@ def from_hf_config(path: str, name: Optional[str] = None) -> ModelConfig:
     if c.get("architecture") == "Dofivik":
         return dofivik_config(name or "dofivik", c["width"], c["vocab"], c["layers"], c["postln_alpha"],
                               c["canon"]["taps"], c["norm"]["eps"], int(c.get("max_position", 32768)))
+    if c.get("architecture") == "Vizonex":
+        return vizonex_config(name or "vizonex", c["width"], c["vocab"], c["layers"], c["canon"]["taps"],
+                              c["norm"]["eps"], int(c["max_positions"]))
     mt = c.get("model_type", "llama")
     eos = c.get("eos_token_id", 2)
     eos = eos if isinstance(eos, list) else [eos]

@@ -23,8 +23,7 @@ taps - 1 inputs of every convolution and the delta-rule states.
 from __future__ import annotations
 
 import math
-from dataclasses import dataclass, field
-from typing import Dict, List, Optional
+from typing import Dict, Optional
 
 import torch
 import torch.nn as nn
@@ -34,6 +33,7 @@ from ..ops import seqmix as sq
 from ..parallel.state import get_state
 from .base import AttnMeta
 from .config import ModelConfig
+from .seq_cache import LayerCache, SeqCache
 
 
 def _p(t):
@@ -42,33 +42,6 @@ def _p(t):
 
 def _softplus(v: float) -> float:
     return v if v > 30 else math.log1p(math.exp(v))
-
-
-@dataclass
-class LayerCache:
-    latent: Optional[torch.Tensor] = None   # [num_blocks * block_size, kv_rank + rot_dim] (owner's tensor)
-    conv1: Optional[torch.Tensor] = None    # fp32 [slots, taps - 1, width]
-    conv2: Optional[torch.Tensor] = None
-    delta: Optional[torch.Tensor] = None    # fp32 [slots, heads, dim, dim]
-
-
-@dataclass
-class SeqCache:
-    """Pages + per-slot state of every layer (the model's share of the engine's cache)."""
-    layers: List[LayerCache] = field(default_factory=list)
-    block_size: int = 16
-
-    def tensors(self):
-        seen, out = set(), []
-        for L in self.layers:
-            for t in (L.latent, L.conv1, L.conv2, L.delta):
-                if t is not None and t.data_ptr() not in seen and t.numel():
-                    seen.add(t.data_ptr())
-                    out.append(t)
-        return out
-
-    def nbytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in self.tensors())
 
 
 class LatentAttentionMixer(nn.Module):

@@ -22,10 +22,11 @@ from .config import ModelConfig, get_config
 from .dofivik import DofivikForCausalLM
 from .gpt2 import GPT2ForCausalLM
 from .llama import LlamaForCausalLM
+from .vizonex import VizonexForCausalLM
 
 
 def model_class(cfg: ModelConfig):
-    return {"gpt2": GPT2ForCausalLM, "dofivik": DofivikForCausalLM}.get(cfg.arch, LlamaForCausalLM)
+    return {"gpt2": GPT2ForCausalLM, "dofivik": DofivikForCausalLM, "vizonex": VizonexForCausalLM}.get(cfg.arch, LlamaForCausalLM)
 
 
 def _resolve_shapes(cfg: ModelConfig, checkpoint: str) -> None:
@@ -120,6 +121,8 @@ def load_checkpoint(model, path: str) -> None:
         _load_gpt2(model, r)
     elif cfg.arch == "dofivik":
         _load_dofivik(model, r)
+    elif cfg.arch == "vizonex":
+        _load_vizonex(model, r)
     else:
         _load_llama(model, r)
 
@@ -231,6 +234,67 @@ def _load_dofivik(m, r: _Reader):
     m.finalize_weights()
 
 
+def _vizonex_tensors(m):
+    """(checkpoint name, parameter, index of a fused / stacked parameter or None) for every tensor."""
+    out = [("embed", m.embed, None), ("pos", m.pos, None), ("head", m.head, None), ("final.norm", m.final_norm, None)]
+
+    def glu(pre, mod):
+        F_ = mod.ff
+        return [(pre + "gate", mod.gate_up, slice(0, F_)), (pre + "up", mod.gate_up, slice(F_, 2 * F_)),
+                (pre + "down", mod.down, None)]
+    for i, L in enumerate(m.layers):
+        b, x = f"l{i}.", L.mix
+        out += [(b + "norm1", L.norm1, None), (b + "ls1", L.ls1, None), (b + "canon1", L.canon1, None)]
+        if L.kind == "attention":
+            out += [(b + "mix.q", x.qkv, slice(0, x.nq)), (b + "mix.k", x.qkv, slice(x.nq, x.nq + x.nk)),
+                    (b + "mix.v", x.qkv, slice(x.nq + x.nk, x.nq + x.nk + x.nv)), (b + "mix.q.norm", x.q_norm, None),
+                    (b + "mix.k.norm", x.k_norm, None), (b + "mix.temp", x.temp, None), (b + "mix.sink", x.sink, None),
+                    (b + "mix.o", x.o, None)]
+        else:
+            out += [(b + "mix.in", x.in_proj, None), (b + "mix.conv", x.conv_w, None), (b + "mix.conv.b", x.conv_b, None),
+                    (b + "mix.dt_bias", x.dt_bias, None), (b + "mix.A_log", x.A_log, None), (b + "mix.D", x.D, None),
+                    (b + "mix.norm", x.norm, None), (b + "mix.o", x.o, None)]
+        if L.mlp is None:
+            continue
+        out.append((b + "ls2", L.ls2, None))
+        if not L.moe:
+            out += glu(b + "mlp.", L.mlp)
+            continue
+        F_ = L.mlp.ff
+        out += [(b + "mlp.router", L.mlp.router, None), (b + "mlp.correction", L.mlp.correction, None)]
+        for e in range(L.mlp.E):
+            out += [(f"{b}mlp.e{e}.gate", L.mlp.w13, (e, slice(0, F_))), (f"{b}mlp.e{e}.up", L.mlp.w13, (e, slice(F_, 2 * F_))),
+                    (f"{b}mlp.e{e}.down", L.mlp.w2, e)]
+        if L.mlp.shared is not None:
+            out += glu(b + "mlp.shared.", L.mlp.shared)
+    return out
+
+
+def _load_vizonex(m, r: _Reader):
+    """Tensors `embed`, `pos`, `head`, `final.norm`, `l<i>.<norm1|ls1|ls2|canon1>`, `l<i>.mix.*`, `l<i>.mlp.*`
+    ([out, in] matrices). q / k / v and gate / up are fused row-wise, the experts stacked, on load."""
+    for name, p, idx in _vizonex_tensors(m):
+        src = r.get(name)
+        dst = p.data if idx is None else p.data[idx]
+        if tuple(dst.shape) != tuple(src.shape):
+            raise ValueError(f"shape mismatch for {name}: model {tuple(dst.shape)} vs checkpoint {tuple(src.shape)}")
+        dst.copy_(src.to(dst.dtype))
+
+
+def _save_vizonex(model, path: str) -> None:
+    from safetensors.torch import save_file
+    cfg = model.cfg
+    t = {}
+    for name, p, idx in _vizonex_tensors(model):
+        v = p.data if idx is None else p.data[idx]
+        t[name] = v.detach().to(torch.bfloat16).contiguous().cpu()
+    save_file(t, os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump({"architecture": "Vizonex", "width": cfg.hidden_size, "vocab": cfg.vocab_size,
+                   "layers": cfg.layer_specs, "canon": {"taps": cfg.canon_taps}, "norm": {"eps": cfg.norm_eps},
+                   "max_positions": cfg.max_position}, f, indent=1)
+
+
 def _save_dofivik(model, path: str) -> None:
     from safetensors.torch import save_file
     cfg = model.cfg
@@ -258,6 +322,8 @@ def save_checkpoint(model, path: str) -> None:
     os.makedirs(path, exist_ok=True)
     if cfg.arch == "dofivik":
         return _save_dofivik(model, path)
+    if cfg.arch == "vizonex":
+        return _save_vizonex(model, path)
     t: Dict[str, torch.Tensor] = {}
     if cfg.arch == "gpt2":
         t["transformer.wte.weight"] = model.wte

@@ -45,17 +45,27 @@ def _i32(t: torch.Tensor) -> torch.Tensor:
 
 
 # ---------------------------------------------------------------------------- embedding
-def embed_rows(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """fp32 rows table[ids] (zero rows for ids outside the table)."""
+def embed_rows(ids: torch.Tensor, table: torch.Tensor, pos_table: Optional[torch.Tensor] = None,
+               positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 rows table[ids] (zero rows for ids outside the table); with `pos_table` the learned vector
+    pos_table[positions] is added (unscaled)."""
     V, W = table.shape
     if not native_device(table):
         ok = (ids >= 0) & (ids < V)
         out = table[ids.long().clamp(0, V - 1)].float()
         out[~ok] = 0
+        if pos_table is not None:
+            pk = (positions >= 0) & (positions < pos_table.shape[0])
+            add = pos_table[positions.long().clamp(0, pos_table.shape[0] - 1)].float()
+            add[~pk] = 0
+            out = out + add
         return out
     out = torch.empty(ids.shape[0], W, dtype=torch.float32, device=table.device)
+    if pos_table is not None:
+        assert pos_table.dtype == table.dtype and pos_table.shape[1] == W and pos_table.is_contiguous()
     mixers().embed_rows(_i32(ids).data_ptr(), table.data_ptr(), is_f32(table), out.data_ptr(), ids.shape[0], W, V,
-                        stream_ptr())
+                        _p(pos_table), _i32(positions).data_ptr() if pos_table is not None else 0,
+                        pos_table.shape[0] if pos_table is not None else 0, stream_ptr())
     return out
 
 
@@ -87,6 +97,45 @@ def causal_conv_residual(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor, 
         y = x[a:b].clone()
         for j in range(taps):
             y += w[:, j] * ext[j:j + b - a]
+        out[a:b] = y.to(out_dtype)
+        if nh:
+            state[slots[s]] = ext[-nh:]
+    return out
+
+
+def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, sm: SeqMeta,
+                out_dtype: torch.dtype, residual: bool = False, silu: bool = False) -> torch.Tensor:
+    """Causal depthwise convolution over time of a row-strided activation block x [T, C] (float32 or
+    bfloat16): out_t = [x_t] + bias + sum_j w[:, j] x_(t - taps + 1 + j), optionally through silu; zeros
+    before a sequence's start. state fp32 [slots, taps - 1, C] holds each sequence's last taps - 1 raw
+    inputs and is updated."""
+    T, C = x.shape
+    taps = w.shape[1]
+    out = torch.empty(T, C, dtype=out_dtype, device=x.device)
+    if native_device(x):
+        assert x.stride(1) == 1 and w.dtype == torch.float32 and w.is_contiguous() and w.shape[0] == C
+        assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (taps - 1, C)
+        mixers().causal_conv(x.data_ptr(), is_f32(x), x.stride(0), w.data_ptr(), _p(bias), state.data_ptr(),
+                             _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(), _i32(sm.slots).data_ptr(),
+                             out.data_ptr(), is_f32(out), sm.num_seqs, sm.max_q, C, taps, residual, silu, stream_ptr())
+        return out
+    nh = taps - 1
+    qsl, sl, slots = sm.qsl.tolist(), sm.seq_lens.tolist(), sm.slots.tolist()
+    xf = x.float()
+    for s in range(sm.num_seqs):
+        a, b = qsl[s], qsl[s + 1]
+        if slots[s] < 0 or b <= a:
+            continue
+        ctx = sl[s] - (b - a)
+        hist = state[slots[s]] if ctx > 0 else torch.zeros(nh, C)
+        ext = torch.cat([hist, xf[a:b]], 0)
+        y = xf[a:b].clone() if residual else torch.zeros(b - a, C)
+        if bias is not None:
+            y = y + bias
+        for j in range(taps):
+            y = y + w[:, j] * ext[j:j + b - a]
+        if silu:
+            y = y * torch.sigmoid(y)
         out[a:b] = y.to(out_dtype)
         if nh:
             state[slots[s]] = ext[-nh:]
@@ -331,4 +380,270 @@ def tanh_cols(x: torch.Tensor, off: int, n: int) -> torch.Tensor:
         return torch.tanh(x[:, off:off + n].float()).to(x.dtype)
     out = torch.empty(T, n, dtype=x.dtype, device=x.device)
     mixers().tanh_cols(x.data_ptr() + off * x.element_size(), is_f32(x), x.stride(0), out.data_ptr(), T, n, stream_ptr())
+    return out
+
+
+# ---------------------------------------------------------------------------- parallel-block residual + next norm
+def residual_norm(x: torch.Tensor, y1: Optional[torch.Tensor], a1: Optional[torch.Tensor], y2: Optional[torch.Tensor],
+                  y3: Optional[torch.Tensor], a2: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], eps: float,
+                  out_dtype: Optional[torch.dtype] = None, want_f32: bool = False):
+    """x <- x + a1 * y1 + a2 * (y2 + y3) in place (x fp32 [T, W]; y1 / y2 activation tensors, y3 fp32; a1 / a2
+    per-channel scales, None = 1; any y may be None), then, with `norm_w`, the RMS norm of the new x:
+    n = x / sqrt(mean(x^2) + eps) * norm_w, returned as (n fp32 or None, n as out_dtype or None)."""
+    T, W = x.shape
+    if not native_device(x):
+        v = x
+        if y1 is not None:
+            v = v + (a1 if a1 is not None else 1.0) * y1.float()
+        if y2 is not None or y3 is not None:
+            f = (y2.float() if y2 is not None else 0.0) + (y3 if y3 is not None else 0.0)
+            v = v + (a2 if a2 is not None else 1.0) * f
+        x.copy_(v)
+        if norm_w is None:
+            return None, None
+        n = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * norm_w
+        return (n if want_f32 else None), (n.to(out_dtype) if out_dtype is not None else None)
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    ys = [y for y in (y1, y2) if y is not None]
+    assert all(y.stride(1) == 1 and y.shape == x.shape for y in ys) and len({y.dtype for y in ys}) <= 1
+    assert y3 is None or (y3.dtype == torch.float32 and y3.is_contiguous() and y3.shape == x.shape)
+    n32 = torch.empty_like(x) if (norm_w is not None and want_f32) else None
+    nact = torch.empty(T, W, dtype=out_dtype, device=x.device) if (norm_w is not None and out_dtype is not None) else None
+    mixers().residual_norm(x.data_ptr(), _p(y1), y1.stride(0) if y1 is not None else 0, _p(a1), _p(y2),
+                           y2.stride(0) if y2 is not None else 0, _p(y3), _p(a2), is_f32(ys[0]) if ys else True,
+                           _p(norm_w), float(eps), _p(n32), _p(nact), is_f32(nact) if nact is not None else True, T, W,
+                           stream_ptr())
+    return n32, nact
+
+
+# ---------------------------------------------------------------------------- grouped-query attention, masked
+MASK_CAUSAL, MASK_WINDOW, MASK_CHUNK = 0, 1, 2
+# XGS_TUNE attn_mfma=0: the general (any size, fp32-capable) kernel for bf16 too (A/B and tests)
+ATTN_MFMA = tune.get_bool("attn_mfma", True)
+
+
+def first_visible(mask: int, size: int, pos: int) -> int:
+    """The first key position a query at `pos` sees: 0 (causal), pos - size + 1 (sliding window), or the
+    start of its chunk of `size` positions counted from the sequence's start (chunked)."""
+    if mask == MASK_WINDOW:
+        return max(0, pos - size + 1)
+    if mask == MASK_CHUNK:
+        return (pos // size) * size
+    return 0
+
+
+def qk_norm_cache(proj: torch.Tensor, nq: int, nk: int, nv: int, wq: Optional[torch.Tensor], wk: Optional[torch.Tensor],
+                  eps: float, sm: SeqMeta, kcache: torch.Tensor, vcache: torch.Tensor) -> torch.Tensor:
+    """From a fused projection row [q (nq) | k (nk) | v (nv)]: q and k are RMS-normed over their WHOLE
+    vectors (all heads at once; weights wq / wk, None = no norm); q is returned [T, nq], k and v go to
+    cache rows slot_mapping[t] (kcache [rows, nk], vcache [rows, nv])."""
+    T = proj.shape[0]
+    q = torch.empty(T, nq, dtype=proj.dtype, device=proj.device)
+    if native_device(proj):
+        assert proj.stride(1) == 1 and kcache.is_contiguous() and vcache.is_contiguous()
+        assert kcache.dtype == vcache.dtype == proj.dtype and kcache.shape[-1] == nk and vcache.shape[-1] == nv
+        mixers().qk_norm_cache(proj.data_ptr(), is_f32(proj), proj.stride(0), nq, nk, nv, _p(wq), _p(wk), float(eps),
+                               _i32(sm.slot_mapping).data_ptr(), q.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), T,
+                               stream_ptr())
+        return q
+    pf = proj.float()
+
+    def nrm(v, w):
+        return v if w is None else v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w
+    q.copy_(nrm(pf[:, :nq], wq).to(proj.dtype))
+    ok = sm.slot_mapping >= 0
+    rows = sm.slot_mapping[ok].long()
+    kcache.view(-1, nk)[rows] = nrm(pf[:, nq:nq + nk], wk)[ok].to(kcache.dtype)
+    vcache.view(-1, nv)[rows] = proj[:, nq + nk:nq + nk + nv][ok].to(vcache.dtype)
+    return q
+
+
+def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, H: int, G: int, dk: int, dv: int,
+                     mask: int, size: int, scale: float, temp: Optional[torch.Tensor], sink: Optional[torch.Tensor],
+                     block_size: int, sm: SeqMeta) -> torch.Tensor:
+    """Softmax attention of H query heads over G cached key/value heads (query head h reads head h // (H / G)).
+    A query at position i sees keys first_visible(mask, size, i) .. i of its own sequence; positions do not
+    enter the scores. score = (q . k) * scale * temp[h]; with `sink` the denominator also holds exp(sink[h]),
+    a term with no key and no value. q [T, H * dk]; caches [rows, G * dk] / [rows, G * dv]; returns [T, H * dv]."""
+    T = q.shape[0]
+    out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    if native_device(q):
+        assert q.is_contiguous() and kcache.is_contiguous() and vcache.is_contiguous()
+        assert kcache.dtype == vcache.dtype == q.dtype
+        bt = _i32(sm.block_tables)
+        if (ATTN_MFMA and q.dtype == torch.bfloat16 and hasattr(mixers(), "masked_attention_mfma")
+                and dk % 32 == 0 and dv % 16 == 0 and dk <= 256 and dv <= 256):
+            mixers().masked_attention_mfma(q.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), bt.data_ptr(), bt.shape[1],
+                                           block_size, _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
+                                           _i32(sm.slots).data_ptr(), _p(temp), _p(sink), out.data_ptr(), T, sm.num_seqs,
+                                           sm.max_q, H, G, dk, dv, int(mask), int(size), float(scale), stream_ptr())
+            return out
+        mixers().masked_attention(q.data_ptr(), is_f32(q), kcache.data_ptr(), vcache.data_ptr(), bt.data_ptr(),
+                                  bt.shape[1], block_size, _i32(sm.positions).data_ptr(), _i32(sm.token_seq).data_ptr(),
+                                  _p(temp), _p(sink), out.data_ptr(), T, H, G, dk, dv, int(mask), int(size), float(scale),
+                                  stream_ptr())
+        return out
+    kr, vr = kcache.view(-1, G, dk), vcache.view(-1, G, dv)
+    qf = q.float().view(T, H, dk)
+    rep = H // G
+    tseq, pos = sm.token_seq.tolist(), sm.positions.tolist()
+    tmp = temp if temp is not None else torch.ones(H)
+    for t in range(T):
+        s = tseq[t]
+        if s < 0:
+            out[t] = 0
+            continue
+        keys = torch.arange(first_visible(mask, size, pos[t]), pos[t] + 1)
+        idx = sm.block_tables[s][(keys // block_size).long()].long() * block_size + keys % block_size
+        kk = kr[idx].float().repeat_interleave(rep, 1)   # [n, H, dk]
+        vv = vr[idx].float().repeat_interleave(rep, 1)
+        sc = torch.einsum("hd,nhd->hn", qf[t], kk) * (scale * tmp)[:, None]
+        if sink is not None:
+            sc = torch.cat([sc, sink[:, None]], 1)
+        p = torch.softmax(sc, -1)[:, :keys.numel()]
+        out[t] = torch.einsum("hn,nhd->hd", p, vv).reshape(H * dv).to(out.dtype)
+    return out
+
+
+# ---------------------------------------------------------------------------- state-space recurrence
+def ssm_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, A_log: torch.Tensor, D: torch.Tensor,
+             state: torch.Tensor, H: int, G: int, N: int, P: int, sm: SeqMeta) -> torch.Tensor:
+    """Per head h (group h // (H / G)), with x / B / C the column blocks [H P | G N | G N] of `xbc` and
+    dt = softplus(dt_raw + dt_bias) (no clamp):  S <- exp(-exp(A_log_h) dt) S + dt B x^T  (S is N x P),
+    y = S^T C + D_h x. state fp32 [slots, H, N, P] is carried and updated. Returns y fp32 [T, H * P]."""
+    T = xbc.shape[0]
+    y = torch.empty(T, H * P, dtype=torch.float32, device=xbc.device)
+    if native_device(xbc):
+        assert xbc.stride(1) == 1 and dt_raw.stride(1) == 1 and dt_raw.dtype == xbc.dtype
+        assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, N, P)
+        mixers().ssm_scan(xbc.data_ptr(), is_f32(xbc), xbc.stride(0), dt_raw.data_ptr(), dt_raw.stride(0),
+                          dt_bias.data_ptr(), A_log.data_ptr(), D.data_ptr(), state.data_ptr(), _i32(sm.qsl).data_ptr(),
+                          _i32(sm.seq_lens).data_ptr(), _i32(sm.slots).data_ptr(), y.data_ptr(), sm.num_seqs, H, G, N, P,
+                          stream_ptr())
+        return y
+    xf = xbc.float()
+    x = xf[:, :H * P].view(T, H, P)
+    B = xf[:, H * P:H * P + G * N].view(T, G, N).repeat_interleave(H // G, 1)
+    C = xf[:, H * P + G * N:H * P + 2 * G * N].view(T, G, N).repeat_interleave(H // G, 1)
+    dt = torch.nn.functional.softplus(dt_raw.float()[:, :H] + dt_bias, threshold=20.0)
+    dec = torch.exp(-torch.exp(A_log) * dt)
+    qsl, sl, slots = sm.qsl.tolist(), sm.seq_lens.tolist(), sm.slots.tolist()
+    for s in range(sm.num_seqs):
+        lo, hi = qsl[s], qsl[s + 1]
+        if slots[s] < 0 or hi <= lo:
+            continue
+        S = state[slots[s]].clone() if sl[s] - (hi - lo) > 0 else torch.zeros(H, N, P)
+        for t in range(lo, hi):
+            S = dec[t][:, None, None] * S + (dt[t][:, None] * B[t])[:, :, None] * x[t][:, None, :]
+            y[t] = (torch.einsum("hnp,hn->hp", S, C[t]) + D[:, None] * x[t]).reshape(H * P)
+        state[slots[s]] = S
+    return y
+
+
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, eps: float, groups: int,
+                     out_dtype: torch.dtype) -> torch.Tensor:
+    """v = y * silu(z); each of `groups` equal parts of a row divided by its own root mean square; times w.
+    y fp32 [T, n]; z [T, n] (row-strided activation)."""
+    T, n = y.shape
+    if not native_device(y):
+        zf = z.float()
+        v = (y * zf * torch.sigmoid(zf)).view(T, groups, n // groups)
+        v = (v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, n)
+        return (v * w).to(out_dtype)
+    out = torch.empty(T, n, dtype=out_dtype, device=y.device)
+    assert y.is_contiguous() and z.stride(1) == 1 and z.dtype == out_dtype
+    mixers().gated_group_norm(y.data_ptr(), z.data_ptr(), is_f32(z), z.stride(0), w.data_ptr(), float(eps),
+                              out.data_ptr(), T, n, groups, stream_ptr())
+    return out
+
+
+# ---------------------------------------------------------------------------- gated feed-forward, routed experts
+GLU_GELU_TANH, GLU_CLAMPED = 0, 1
+# XGS_TUNE moe_mfma=0: the general grouped GEMM for bf16 too (A/B and tests)
+MOE_MFMA = tune.get_bool("moe_mfma", True)
+
+
+def _glu_ref(g, u, kind, limit, alpha):
+    if kind == GLU_GELU_TANH:
+        return 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g ** 3))) * u
+    g = g.clamp(max=limit)
+    u = u.clamp(-limit, limit)
+    return g * torch.sigmoid(alpha * g) * (u + 1.0)
+
+
+def glu_act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.702) -> torch.Tensor:
+    """Rows [gate (F) | up (F)] -> [F]: GLU_GELU_TANH: gelu_tanh(gate) * up; GLU_CLAMPED: with g = min(gate, limit),
+    u = clamp(up, -limit, limit): g * sigmoid(alpha g) * (u + 1)."""
+    T, F2 = x.shape
+    F_ = F2 // 2
+    if not native_device(x):
+        xf = x.float()
+        return _glu_ref(xf[:, :F_], xf[:, F_:], kind, limit, alpha).to(x.dtype)
+    assert x.stride(1) == 1
+    out = torch.empty(T, F_, dtype=x.dtype, device=x.device)
+    mixers().glu_act(x.data_ptr(), is_f32(x), x.stride(0), out.data_ptr(), T, F_, int(kind), float(limit), float(alpha),
+                     stream_ptr())
+    return out
+
+
+def grouped_router(logits: torch.Tensor, correction: Optional[torch.Tensor], count: int, keep: int, top: int,
+                   scale: float):
+    """fp32 router logits [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]). Scores are
+    sigmoid(logits); experts are CHOSEN by score + correction, restricted to the `keep` best of `count`
+    groups of neighbouring experts (a group scores the sum of its two largest choice scores; experts of
+    other groups count as -inf), and WEIGHTED by score * scale (no correction, no renormalisation)."""
+    T, E = logits.shape
+    if not native_device(logits):
+        s = torch.sigmoid(logits.float())
+        c = s + (correction if correction is not None else 0.0)
+        per = E // count
+        gsc = c.view(T, count, per).topk(min(2, per), -1).values.sum(-1)
+        kept = torch.zeros(T, count, dtype=torch.bool)
+        kept.scatter_(1, gsc.topk(keep, -1).indices, True)
+        c = c.masked_fill(~kept.repeat_interleave(per, 1), float("-inf"))
+        ids = c.topk(top, -1).indices
+        return ids.to(torch.int32), s.gather(1, ids) * scale
+    assert logits.dtype == torch.float32 and logits.is_contiguous()
+    ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    mixers().grouped_router(logits.data_ptr(), _p(correction), T, E, int(count), int(keep), int(top), float(scale),
+                            ids.data_ptr(), wts.data_ptr(), stream_ptr())
+    return ids, wts
+
+
+def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, kind: int,
+                   limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """sum_j wts[t, j] * W2[e] glu(W13[e] h_t), e = ids[t, j]. w13 [E, 2 F, K] holds each expert's gate rows then
+    its up rows, w2 [E, W, F]. Returns fp32 [T, W] (a sum in a fixed order per row)."""
+    T, K = h.shape
+    E, F2, _ = w13.shape
+    F_, W, top = F2 // 2, w2.shape[1], ids.shape[1]
+    if not native_device(h):
+        out = torch.zeros(T, W)
+        hf = h.float()
+        for e in range(E):
+            tt, jj = torch.nonzero(ids == e, as_tuple=True)
+            if tt.numel() == 0:
+                continue
+            gu = (hf[tt] @ w13[e].float().t()).to(h.dtype).float()
+            a = _glu_ref(gu[:, :F_], gu[:, F_:], kind, limit, alpha).to(h.dtype).float()
+            out.index_add_(0, tt, (a @ w2[e].float().t()) * wts[tt, jj][:, None])
+        return out
+    M = mixers()
+    tm = M.MOE_TILE_M
+    assert h.is_contiguous() and w13.is_contiguous() and w2.is_contiguous() and w13.dtype == w2.dtype == h.dtype
+    pairs = T * top
+    cap = (pairs + E * (tm - 1) + tm - 1) // tm * tm
+    dev = h.device
+    meta = torch.empty(cap + cap // tm + pairs, dtype=torch.int32, device=dev)
+    rows, tile_e, dest = meta[:cap], meta[cap:cap + cap // tm], meta[cap + cap // tm:]
+    M.moe_align(_i32(ids).data_ptr(), pairs, E, cap, rows.data_ptr(), tile_e.data_ptr(), dest.data_ptr(), stream_ptr())
+    act = torch.empty(cap, F_, dtype=h.dtype, device=dev)
+    M.grouped_gemm(h.data_ptr(), is_f32(h), h.stride(0), w13.data_ptr(), rows.data_ptr(), tile_e.data_ptr(), cap, top, F_,
+                   K, True, act.data_ptr(), int(kind), float(limit), float(alpha), MOE_MFMA, stream_ptr())
+    y = torch.empty(cap, W, dtype=torch.float32, device=dev)
+    M.grouped_gemm(act.data_ptr(), is_f32(act), F_, w2.data_ptr(), rows.data_ptr(), tile_e.data_ptr(), cap, top, W, F_,
+                   False, y.data_ptr(), 0, 0.0, 0.0, MOE_MFMA, stream_ptr())
+    out = torch.empty(T, W, dtype=torch.float32, device=dev)
+    M.moe_combine(y.data_ptr(), dest.data_ptr(), wts.data_ptr(), T, top, W, out.data_ptr(), stream_ptr())
     return out
