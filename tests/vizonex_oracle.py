@@ -46,27 +46,34 @@ def shifted_conv(h, w, bias=None):
 
 
 # ------------------------------------------------------------------------------ attention in chunks, with a sink
+def chunk_softmax(q, k, v, size, scale, temp, sink):
+    """q [T, H, dk], k [T, G, dk], v [T, G, dv] of one sequence -> [T, H, dv]. Query i reads keys j <= i of its
+    own chunk floor(i / size); the denominator carries exp(sink_h) besides the keys' terms."""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    out = torch.zeros(T, H, v.shape[2], dtype=F64)
+    for hd in range(H):
+        g = hd // (H // G)
+        for i in range(T):
+            lo = (i // size) * size
+            s = (k[lo:i + 1, g] @ q[i, hd]) * scale * temp[hd]
+            top = torch.maximum(s.max(), sink[hd])
+            e = torch.exp(s - top)
+            out[i, hd] = (e[:, None] * v[lo:i + 1, g]).sum(0) / (e.sum() + torch.exp(sink[hd] - top))
+    return out
+
+
 def chunk_attention(Wt, pre, m, h, eps):
     """Whole-vector query / key norms, no positional rotation, per-head temperature, keys of the
     query's own chunk only (chunks of m.mask.size counted from t = 0), and one extra term
     exp(sink_h) in the softmax denominator that carries no value."""
     T = h.shape[0]
     H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    size, scale = int(m["mask"]["size"]), float(m["scale"])
     q = unit_rms(h @ Wt[pre + "q"].T, eps) * Wt[pre + "q.norm"]
     k = unit_rms(h @ Wt[pre + "k"].T, eps) * Wt[pre + "k.norm"]
     v = h @ Wt[pre + "v"].T
-    q, k, v = q.reshape(T, H, dk), k.reshape(T, G, dk), v.reshape(T, G, dv)
-    out = torch.zeros(T, H, dv, dtype=F64)
-    for hd in range(H):
-        g = hd // (H // G)
-        for i in range(T):
-            lo = (i // size) * size
-            s = (k[lo:i + 1, g] @ q[i, hd]) * scale * Wt[pre + "temp"][hd]
-            sink = Wt[pre + "sink"][hd]
-            top = torch.maximum(s.max(), sink)
-            e = torch.exp(s - top)
-            out[i, hd] = (e[:, None] * v[lo:i + 1, g]).sum(0) / (e.sum() + torch.exp(sink - top))
+    out = chunk_softmax(q.reshape(T, H, dk), k.reshape(T, G, dk), v.reshape(T, G, dv), int(m["mask"]["size"]),
+                        float(m["scale"]), Wt[pre + "temp"], Wt[pre + "sink"])
     return out.reshape(T, H * dv) @ Wt[pre + "o"].T
 
 
@@ -111,15 +118,15 @@ def clamped_expert(Wt, pre, h, limit):
     return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ Wt[pre + "down"].T
 
 
-def route(Wt, pre, r, h):
-    """Chosen experts and their weights for every row of h: lists of (expert, weight)."""
+def route_scores(z, correction, r):
+    """Router logits z [T, E] -> per row the chosen experts and their weights: lists of (expert, weight)."""
     E, top = r["experts"], r["top"]
     count, keep = r["groups"]["count"], r["groups"]["keep"]
-    s = torch.sigmoid(h @ Wt[pre + "router"].T)
-    pick = s + Wt[pre + "correction"]
+    s = torch.sigmoid(z)
+    pick = s + correction
     per = E // count
     chosen = []
-    for t in range(h.shape[0]):
+    for t in range(z.shape[0]):
         gs = []
         for g in range(count):
             part = sorted(pick[t, g * per:(g + 1) * per].tolist(), reverse=True)
@@ -129,6 +136,10 @@ def route(Wt, pre, r, h):
         cand.sort(key=lambda e: -float(pick[t, e]))
         chosen.append([(e, float(s[t, e]) * r["scale"]) for e in cand[:top]])
     return chosen
+
+
+def route(Wt, pre, r, h):
+    return route_scores(h @ Wt[pre + "router"].T, Wt[pre + "correction"], r)
 
 
 def moe_ff(Wt, pre, mlp, h):
