@@ -73,6 +73,12 @@ def parse():
     ap.add_argument("--dofivik-prompts", type=int, default=4, help="prompts in the one prefill step")
     ap.add_argument("--dofivik-context", type=int, default=1024, help="context length of the decoding rows")
     ap.add_argument("--dofivik-only", default=None, choices=["dofivik", "llama"])
+    ap.add_argument("--vizonex", action="store_true",
+                    help="instead of the headline: prefill and decode tokens/s of Vizonex beside a Mixtral-type model "
+                         "and a Llama of equal layer sizes (bench/vizonex_bench.py; --prompt-len, --concurrency = decode "
+                         "batch, --steps, --warmup, --dofivik-prompts, --dofivik-context apply)")
+    ap.add_argument("--vizonex-sizes", default="1b-class,8b-class")
+    ap.add_argument("--vizonex-only", default=None, choices=["vizonex", "mixtral", "llama"])
     return ap.parse_args()
 
 
@@ -167,11 +173,12 @@ def preflight(st, world: int, tp: int, dev, eng) -> dict:
 
 def main():
     a = parse()
-    if a.dofivik:
+    if a.dofivik or a.vizonex:
         import importlib.util
         here = os.path.dirname(os.path.abspath(__file__))
         sys.path.insert(0, here)
-        spec = importlib.util.spec_from_file_location("dofivik_bench", os.path.join(here, "bench", "dofivik_bench.py"))
+        which = "dofivik_bench" if a.dofivik else "vizonex_bench"
+        spec = importlib.util.spec_from_file_location(which, os.path.join(here, "bench", which + ".py"))
         mod = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(mod)
         return mod.run(a)

@@ -162,6 +162,158 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
   }
 }
 
+
+// ------------------------------------------------------------------ matrix-core form (bf16, dk % 32 == 0, dv % 16 == 0)
+// A wave owns 16 query slots: 16 consecutive tokens of one sequence x one query head. The 4 waves of a
+// workgroup are RH query heads of one key/value head x 4 / RH token tiles, so a tile of 64 keys (K rows and
+// V rows, staged once in LDS) serves all of them. S^T = K Q^T on v_mfma_f32_16x16x32_bf16: the accumulator
+// holds, per lane, 16 keys of ONE slot, and packed to bf16 it is the B operand of O^T += V^T P^T, whose A
+// operand (V^T) is a transposed LDS read of the staged V rows.
+constexpr int kKT = 64;
+
+template <int NKK_MAX, int NMT_MAX>
+__global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
+    const int32_t* __restrict__ block_tables, int bt_width, int bs, const int32_t* __restrict__ qsl,
+    const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots, const float* __restrict__ temp,
+    const float* __restrict__ sink, bf16* __restrict__ out, int H, int G, int dk, int dv, int mask, int size, float scale,
+    int RH) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  const int LDK = dk + 8, LDV = dv + 8;
+  uint16_t* ktile = lds;                 // [kKT][LDK]
+  uint16_t* vtile = lds + kKT * LDK;     // [kKT][LDV]
+  const int s = blockIdx.z;
+  const int q0 = qsl[s], qn = qsl[s + 1] - q0;
+  if (slots[s] < 0 || qn <= 0) return;
+  const int tpb = 4 / RH;                // token tiles per workgroup
+  const int t0 = blockIdx.x * 16 * tpb;
+  if (t0 >= qn) return;
+  const int rep = H / G;
+  const int hblocks = (rep + RH - 1) / RH;
+  const int g = blockIdx.y / hblocks, hb = blockIdx.y % hblocks;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int li = lane & 15, kg = lane >> 4;
+  const int hr = hb * RH + wave % RH;                // head within the group
+  const int tok = t0 + (wave / RH) * 16 + li;        // this lane's slot: token within the sequence's rows
+  const bool wave_on = hr < rep && t0 + (wave / RH) * 16 < qn;
+  const bool valid = wave_on && tok < qn;
+  const int head = g * rep + min(hr, rep - 1);
+  const int ctx = seq_lens[s] - qn;
+  const int pos_q = ctx + min(tok, qn - 1);
+  const int lo_q = first_visible(mask, size, pos_q);
+  const int nkk = dk / 32, nmt = dv / 16;
+  // keys any slot of this workgroup can see
+  const int kmin = first_visible(mask, size, ctx + t0);
+  const int pos_last = ctx + min(qn, t0 + 16 * tpb) - 1;
+  const int32_t* bt = block_tables + (int64_t)s * bt_width;
+
+  xgk::bf16x8_t qf[NKK_MAX];
+#pragma unroll
+  for (int kk = 0; kk < NKK_MAX; ++kk) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (kk < nkk && valid) v = xgk::ld16(q + ((int64_t)(q0 + tok) * H + head) * dk + kk * 32 + kg * 8);
+    qf[kk] = xgk::as_frag(v);
+  }
+  const float sc_h = scale * (temp ? temp[head] : 1.f);
+  xgk::f32x4_t o[NMT_MAX];
+#pragma unroll
+  for (int mt = 0; mt < NMT_MAX; ++mt) o[mt] = xgk::f32x4_t{0.f, 0.f, 0.f, 0.f};
+  // the sink starts the running softmax: weight exp(sink - m) = 1 with no value behind it
+  float m = sink ? sink[head] : -INFINITY, l = sink ? 1.f : 0.f;
+
+  const int srow = threadIdx.x >> 2, squad = threadIdx.x & 3;
+  for (int k0 = kmin; k0 <= pos_last; k0 += kKT) {
+    __syncthreads();
+    {
+      const int kabs = k0 + srow;
+      const bool ok = kabs <= pos_last;
+      const int64_t row = ok ? (int64_t)bt[kabs / bs] * bs + kabs % bs : 0;
+      const bf16* ks = kcache + (row * G + g) * dk;
+      const bf16* vs = vcache + (row * G + g) * dv;
+      for (int ch = squad; ch * 8 < dk; ch += 4)
+        xgk::st16(ktile + srow * LDK + ch * 8, ok ? xgk::ld16(ks + ch * 8) : make_uint4(0, 0, 0, 0));
+      for (int ch = squad; ch * 8 < dv; ch += 4)
+        xgk::st16(vtile + srow * LDV + ch * 8, ok ? xgk::ld16(vs + ch * 8) : make_uint4(0, 0, 0, 0));
+    }
+    __syncthreads();
+    if (!wave_on) continue;
+    xgk::f32x4_t sacc[4];
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      sacc[n] = xgk::f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < NKK_MAX; ++kk)
+        if (kk < nkk)
+          sacc[n] = xgk::mfma16x16x32(xgk::as_frag(xgk::ld16(ktile + (n * 16 + li) * LDK + kk * 32 + kg * 8)), qf[kk],
+                                      sacc[n]);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int kabs = k0 + n * 16 + kg * 4 + r;
+        float v = sacc[n][r] * sc_h;
+        if (!valid || kabs > pos_q || kabs < lo_q) v = -INFINITY;
+        sacc[n][r] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = (m_new == -INFINITY || m == -INFINITY) ? (m == -INFINITY ? 0.f : 1.f) : __expf(m - m_new);
+    float rs = 0.f;
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = m_new == -INFINITY ? 0.f : __expf(sacc[n][r] - m_new);
+        sacc[n][r] = p;
+        rs += p;
+      }
+    rs += __shfl_xor(rs, 16, 64);
+    rs += __shfl_xor(rs, 32, 64);
+    l = l * alpha + rs;
+    m = m_new;
+#pragma unroll
+    for (int mt = 0; mt < NMT_MAX; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[mt][r] *= alpha;
+    // O^T += V^T . P^T over two 32-key halves (keys in the order the score accumulator holds them)
+#pragma unroll
+    for (int sc = 0; sc < 2; ++sc) {
+      uint4 pb;
+      pb.x = xgk::pack2(sacc[2 * sc][0], sacc[2 * sc][1]);
+      pb.y = xgk::pack2(sacc[2 * sc][2], sacc[2 * sc][3]);
+      pb.z = xgk::pack2(sacc[2 * sc + 1][0], sacc[2 * sc + 1][1]);
+      pb.w = xgk::pack2(sacc[2 * sc + 1][2], sacc[2 * sc + 1][3]);
+      const xgk::bf16x8_t pfrag = xgk::as_frag(pb);
+      const int qq = li >> 2, pp = li & 3;
+      const int r0 = sc * 32 + 4 * kg + qq, r1 = r0 + 16;
+#pragma unroll
+      for (int mt = 0; mt < NMT_MAX; ++mt)
+        if (mt < nmt) {
+          const xgk::bf16x4_t a0 = xgk::lds_read_tr16(vtile + r0 * LDV + mt * 16 + 4 * pp);
+          const xgk::bf16x4_t a1 = xgk::lds_read_tr16(vtile + r1 * LDV + mt * 16 + 4 * pp);
+          const xgk::bf16x8_t vfrag = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+          o[mt] = xgk::mfma16x16x32(vfrag, pfrag, o[mt]);
+        }
+    }
+  }
+  if (valid) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16* op = out + ((int64_t)(q0 + tok) * H + head) * dv;
+#pragma unroll
+    for (int mt = 0; mt < NMT_MAX; ++mt)
+      if (mt < nmt) {
+        uint2 w;
+        w.x = xgk::pack2(o[mt][0] * inv, o[mt][1] * inv);
+        w.y = xgk::pack2(o[mt][2] * inv, o[mt][3] * inv);
+        *reinterpret_cast<uint2*>(op + mt * 16 + 4 * kg) = w;
+      }
+  }
+}
+
 // ================================================================== host launchers
 void qk_norm_cache(const void* proj, bool f32, int64_t ld, int nq, int nk, int nv, const float* wq, const float* wk,
                    float eps, const int32_t* slot_mapping, void* q_out, void* kcache, void* vcache, int T_,
@@ -204,6 +356,32 @@ int masked_attention(const void* q, bool f32, const void* kcache, const void* vc
   if (dv <= 256) { XGM_MA(4) }
   XGM_MA(8)
 #undef XGM_MA
+}
+
+
+int masked_attention_mfma(const void* q, const void* kcache, const void* vcache, const int32_t* block_tables, int bt_width,
+                          int bs, const int32_t* qsl, const int32_t* seq_lens, const int32_t* slots, const float* temp,
+                          const float* sink, void* out, int T_, int ns, int max_q, int H, int G, int dk, int dv, int mask,
+                          int size, float scale, hipStream_t st) {
+  if (T_ <= 0 || ns <= 0 || max_q <= 0) return 0;
+  if (G <= 0 || H % G != 0 || dk % 32 != 0 || dv % 16 != 0 || dk > 128 || dv > 128 || mask < 0 || mask > 2 ||
+      (mask != kMaskCausal && size < 1))
+    return -1;
+  const int rep = H / G;
+  const int RH = rep >= 4 ? 4 : rep >= 2 ? 2 : 1;
+  const int tpb = 4 / RH;
+  dim3 grid((max_q + 16 * tpb - 1) / (16 * tpb), G * ((rep + RH - 1) / RH), ns);
+  const size_t lds = (size_t)kKT * (dk + 8 + dv + 8) * sizeof(uint16_t);
+#define XGM_MM(NKK, NMT)                                                                                              \
+  masked_attention_mfma_kernel<NKK, NMT><<<grid, 256, lds, st>>>((const bf16*)q, (const bf16*)kcache,                 \
+                                                                 (const bf16*)vcache, block_tables, bt_width, bs, qsl, \
+                                                                 seq_lens, slots, temp, sink, (bf16*)out, H, G, dk, dv, \
+                                                                 mask, size, scale, RH);                               \
+  return 0;
+  if (dk <= 64 && dv <= 64) { XGM_MM(2, 4) }
+  if (dk <= 128 && dv <= 128) { XGM_MM(4, 8) }
+  return -2;
+#undef XGM_MM
 }
 
 }  // namespace xgm

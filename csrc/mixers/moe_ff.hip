@@ -7,7 +7,7 @@
 //                    `count` equal groups of neighbours, a group scores the sum of its two largest choice
 //                    scores, only experts of the best `keep` groups can be chosen (the others count as
 //                    -inf); the `top` largest choice scores win; weights = score (WITHOUT correction) * scale
-//   moe_align        (token, choice) pairs sorted by expert into tiles of kTileM rows (padded with -1)
+//   moe_align        (token, choice) pairs sorted by expert into tiles of `tm` rows (padded with -1)
 //   grouped_gemm     per tile: rows x expert weights; first GEMM with the gated activation fused,
 //                    second GEMM to fp32 rows
 //   moe_combine      out[t] = sum_j weight[t, j] * y[row of pair (t, j)]   (fixed order: bit-stable)
@@ -20,7 +20,6 @@
 namespace xgm {
 
 constexpr int kGluGeluTanh = 0, kGluClamped = 1;
-constexpr int kTileM = 16;  // rows per expert tile
 
 __device__ __forceinline__ float glu(int kind, float g, float u, float limit, float alpha) {
   if (kind == kGluGeluTanh) {
@@ -116,8 +115,8 @@ __global__ __launch_bounds__(64) void grouped_router_kernel(const float* __restr
 
 // ------------------------------------------------------------------ pairs -> expert tiles (one workgroup)
 __global__ __launch_bounds__(1024) void moe_align_kernel(const int32_t* __restrict__ ids, int pairs, int E, int cap,
-                                                         int32_t* __restrict__ rows, int32_t* __restrict__ tile_expert,
-                                                         int32_t* __restrict__ dest) {
+                                                         int kTileM, int32_t* __restrict__ rows,
+                                                         int32_t* __restrict__ tile_expert, int32_t* __restrict__ dest) {
   extern __shared__ int si[];
   int* cnt = si;          // [E]
   int* off = si + E;      // [E + 1] padded starts
@@ -150,35 +149,36 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int32_t* __restri
 }
 
 // ------------------------------------------------------------------ grouped GEMM, general form
-// Tile = kTileM rows x 64 columns, 256 threads: thread (tr = tid / 16, tc = tid % 16) owns row tr and
+// Tile = 16 rows x 64 columns, 256 threads: thread (tr = tid / 16, tc = tid % 16) owns row tr and
 // columns tc + 16 j. K runs through LDS in chunks of 32. GATED: the weight holds [gate (F rows) | up (F rows)]
-// and the output column f is glu(gate_f, up_f); A rows are gathered through rows[] / top.
+// and the output column f is glu(gate_f, up_f); A rows are gathered through rows[] / top. `tm` = rows per
+// expert tile of the layout (a multiple of 16).
 template <typename T, bool GATED>
 __global__ __launch_bounds__(256) void grouped_gemm_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ Wt,
                                                            const int32_t* __restrict__ rows,
-                                                           const int32_t* __restrict__ tile_expert, int top, int Nout,
-                                                           int K, void* __restrict__ out, int kind, float limit,
+                                                           const int32_t* __restrict__ tile_expert, int tm, int top,
+                                                           int Nout, int K, void* __restrict__ out, int kind, float limit,
                                                            float alpha) {
-  __shared__ float As[kTileM][33];
+  __shared__ float As[16][33];
   __shared__ float Ws[64][33];
   __shared__ float Us[GATED ? 64 : 1][33];
-  const int tile = blockIdx.x;
-  const int e = tile_expert[tile];
+  const int rbase = blockIdx.x * 16;
+  const int e = tile_expert[rbase / tm];
   if (e < 0) return;
   const int n0 = blockIdx.y * 64;
   const int tr = threadIdx.x >> 4, tc = threadIdx.x & 15;
-  const int r = tile * kTileM + tr;
+  const int r = rbase + tr;
   const int pr = rows[r];
   const int64_t wrows = GATED ? 2 * (int64_t)Nout : (int64_t)Nout;
   const T* We = Wt + (int64_t)e * wrows * K;
   float acc[4] = {0.f, 0.f, 0.f, 0.f}, accu[4] = {0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < K; k0 += 32) {
     __syncthreads();
-    for (int i = threadIdx.x; i < kTileM * 32; i += 256) {
+    for (int i = threadIdx.x; i < 16 * 32; i += 256) {
       const int rr = i >> 5, kk = i & 31;
-      const int p2 = rows[tile * kTileM + rr];
+      const int p2 = rows[rbase + rr];
       float v = 0.f;
-      if (p2 >= 0 && k0 + kk < K) v = ldf(A + (int64_t)(GATED ? p2 / top : tile * kTileM + rr) * lda + k0 + kk);
+      if (p2 >= 0 && k0 + kk < K) v = ldf(A + (int64_t)(GATED ? p2 / top : rbase + rr) * lda + k0 + kk);
       As[rr][kk] = v;
     }
     for (int i = threadIdx.x; i < 64 * 32; i += 256) {
@@ -208,61 +208,117 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const T* __restrict__
   }
 }
 
-// ---- matrix-core form (bf16; K % 32 == 0, Nout % 16 == 0): one wave = 16 rows x 16 NT columns,
-// A / B fragments straight from global memory (16 bytes per lane), fp32 accumulators.
+// ---- matrix-core form (bf16; K % 32 == 0, Nout % 16 == 0). A / B fragments come straight from global
+// memory (16 bytes per lane), accumulators are fp32. Two shapes of one kernel:
+//   SPLITK = false (prompt-sized steps, layout tiles of 64 rows): a workgroup owns 16 MT rows x 4 x 16 NT columns,
+//            each wave 16 NT of the columns over the whole K;
+//   SPLITK = true  (few rows per expert, layout tiles of 16 rows): a workgroup owns 16 rows x 16 NT columns, its four
+//            waves a quarter of K each (short dependent load chains, 4 x the workgroups); the partial sums meet in LDS.
 using xgk::as_frag;
 using xgk::f32x4_t;
 using xgk::ld16;
 using xgk::mfma16x16x32;
 
-template <bool GATED, int NT>
+template <bool GATED, int MT, int NT, bool SPLITK>
 __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __restrict__ A, int64_t lda,
                                                                 const bf16* __restrict__ Wt,
                                                                 const int32_t* __restrict__ rows,
                                                                 const int32_t* __restrict__ tile_expert, int top,
                                                                 int Nout, int K, void* __restrict__ out, int kind,
                                                                 float limit, float alpha) {
-  const int tile = blockIdx.x;
+  constexpr int NG = GATED ? NT : 1;
+  __shared__ float red[SPLITK ? 3 : 1][SPLITK ? (NT + NG) : 1][64][4];
+  const int tile = blockIdx.x;          // layout tile of 16 MT rows
   const int e = tile_expert[tile];
   if (e < 0) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n0 = (blockIdx.y * 4 + wave) * 16 * NT;
-  if (n0 >= Nout) return;
+  const int n0 = SPLITK ? blockIdx.y * 16 * NT : (blockIdx.y * 4 + wave) * 16 * NT;
+  if (n0 >= Nout) return;               // (SPLITK: uniform over the workgroup)
   const int l16 = lane & 15, kg = lane >> 4;
   const int64_t wrows = GATED ? 2 * (int64_t)Nout : (int64_t)Nout;
   const bf16* We = Wt + (int64_t)e * wrows * K;
-  const int pa = rows[tile * kTileM + l16];
-  const bf16* arow = A + (int64_t)(GATED ? max(pa, 0) / top : tile * kTileM + l16) * lda + kg * 8;
-  f32x4_t acc[NT], accu[GATED ? NT : 1];
+  const int rbase = tile * 16 * MT;
+  const bf16* arow[MT];
+  bool aok[MT];
 #pragma unroll
-  for (int j = 0; j < NT; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < MT; ++i) {
+    const int pa = rows[rbase + 16 * i + l16];
+    aok[i] = pa >= 0;
+    arow[i] = A + (int64_t)(GATED ? max(pa, 0) / top : rbase + 16 * i + l16) * lda + kg * 8;
+  }
+  f32x4_t acc[MT][NT], accu[MT][NG];
 #pragma unroll
-  for (int j = 0; j < (GATED ? NT : 1); ++j) accu[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    const uint4 av = pa >= 0 ? ld16(arow + k0) : make_uint4(0, 0, 0, 0);
+  for (int i = 0; i < MT; ++i) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < NG; ++j) accu[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  const int kper = SPLITK ? ((K / 32 + 3) / 4) * 32 : K;
+  const int kbeg = SPLITK ? wave * kper : 0, kend = min(K, kbeg + kper);
+#pragma unroll 2
+  for (int k0 = kbeg; k0 < kend; k0 += 32) {
+    uint4 av[MT], bv[NT], uv[NG];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) av[i] = aok[i] ? ld16(arow[i] + k0) : make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-      const int n = n0 + 16 * j + l16;
-      if (n0 + 16 * j < Nout) {  // whole 16-column tiles only (Nout % 16 == 0)
-        // D = A(rows x k) B(k x cols): rows come out along the accumulator's 4 entries x (lane >> 4)
-        acc[j] = mfma16x16x32(as_frag(av), as_frag(ld16(We + (int64_t)n * K + k0 + kg * 8)), acc[j]);
-        if (GATED) accu[j] = mfma16x16x32(as_frag(av), as_frag(ld16(We + (int64_t)(Nout + n) * K + k0 + kg * 8)), accu[j]);
+      const int n = min(n0 + 16 * j, Nout - 16) + l16;  // whole 16-column tiles (Nout % 16 == 0); clamped ones are not stored
+      bv[j] = ld16(We + (int64_t)n * K + k0 + kg * 8);
+      if (GATED) uv[j] = ld16(We + (int64_t)(Nout + n) * K + k0 + kg * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        // D = A (rows x k) B (k x cols): accumulator entry r of lane (l16, kg) is row kg * 4 + r, column l16
+        acc[i][j] = mfma16x16x32(as_frag(av[i]), as_frag(bv[j]), acc[i][j]);
+        if (GATED) accu[i][j] = mfma16x16x32(as_frag(av[i]), as_frag(uv[j]), accu[i][j]);
+      }
+  }
+  if (SPLITK) {  // MT == 1: waves 1..3 hand their partial sums to wave 0
+    if (wave > 0) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[wave - 1][j][lane][r] = acc[0][j][r];
+      if (GATED) {
+#pragma unroll
+        for (int j = 0; j < NG; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) red[wave - 1][NT + j][lane][r] = accu[0][j][r];
+      }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[0][j][r] += red[w][j][lane][r];
+      if (GATED) {
+#pragma unroll
+        for (int j = 0; j < NG; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) accu[0][j][r] += red[w][NT + j][lane][r];
       }
     }
   }
-  // accumulator entry i of lane (l16, kg): row kg * 4 + i, column l16
 #pragma unroll
-  for (int j = 0; j < NT; ++j) {
-    const int n = n0 + 16 * j + l16;
-    if (n0 + 16 * j >= Nout) continue;
+  for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int rr = tile * kTileM + kg * 4 + i;
-      if (rows[rr] < 0) continue;
-      if (GATED) ((bf16*)out)[(int64_t)rr * Nout + n] = f2bf(glu(kind, acc[j][i], accu[j][i], limit, alpha));
-      else ((float*)out)[(int64_t)rr * Nout + n] = acc[j][i];
+    for (int j = 0; j < NT; ++j) {
+      const int n = n0 + 16 * j + l16;
+      if (n0 + 16 * j >= Nout) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int rr = rbase + 16 * i + kg * 4 + r;
+        if (rows[rr] < 0) continue;
+        if (GATED) ((bf16*)out)[(int64_t)rr * Nout + n] = f2bf(glu(kind, acc[i][j][r], accu[i][GATED ? j : 0][r], limit, alpha));
+        else ((float*)out)[(int64_t)rr * Nout + n] = acc[i][j][r];
+      }
     }
-  }
 }
 
 __global__ void moe_combine_kernel(const float* __restrict__ y, const int32_t* __restrict__ dest,
@@ -294,39 +350,41 @@ int grouped_router(const float* logits, const float* corr, int T_, int E, int co
   return 0;
 }
 
-int moe_align(const int32_t* ids, int pairs, int E, int cap, int32_t* rows, int32_t* tile_expert, int32_t* dest,
+int moe_align(const int32_t* ids, int pairs, int E, int cap, int tm, int32_t* rows, int32_t* tile_expert, int32_t* dest,
               hipStream_t st) {
   if (pairs <= 0) return 0;
-  if (E < 1 || E > 4096 || cap % kTileM != 0 || cap < pairs + E * (kTileM - 1)) return -1;
-  moe_align_kernel<<<1, 1024, (2 * E + 1) * sizeof(int), st>>>(ids, pairs, E, cap, rows, tile_expert, dest);
+  if (E < 1 || E > 4096 || tm < 16 || tm % 16 != 0 || cap % tm != 0 || cap < pairs + E * (tm - 1)) return -1;
+  moe_align_kernel<<<1, 1024, (2 * E + 1) * sizeof(int), st>>>(ids, pairs, E, cap, tm, rows, tile_expert, dest);
   return 0;
 }
 
 int grouped_gemm(const void* A, bool f32, int64_t lda, const void* Wt, const int32_t* rows, const int32_t* tile_expert,
-                 int cap, int top, int Nout, int K, bool gated, void* out, int kind, float limit, float alpha, bool mfma,
-                 hipStream_t st) {
+                 int cap, int tm, int top, int Nout, int K, bool gated, void* out, int kind, float limit, float alpha,
+                 bool mfma, hipStream_t st) {
   if (cap <= 0) return 0;
-  if (cap % kTileM != 0 || Nout < 1 || K < 1) return -1;
-  const int tiles = cap / kTileM;
+  if ((tm != 16 && tm != 64) || cap % tm != 0 || Nout < 1 || K < 1) return -1;
   if (!f32 && mfma && K % 32 == 0 && Nout % 16 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)Wt % 16 == 0) {
-    constexpr int NT = 2;
-    dim3 grid(tiles, (Nout + 64 * NT - 1) / (64 * NT));
-    if (gated)
-      grouped_gemm_mfma_kernel<true, NT><<<grid, 256, 0, st>>>((const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top,
-                                                               Nout, K, out, kind, limit, alpha);
-    else
-      grouped_gemm_mfma_kernel<false, NT><<<grid, 256, 0, st>>>((const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert,
-                                                                top, Nout, K, out, kind, limit, alpha);
+#define XGM_GG(GATED, MT, NT, SPLITK, GY)                                                                            \
+  grouped_gemm_mfma_kernel<GATED, MT, NT, SPLITK><<<dim3(cap / tm, GY), 256, 0, st>>>(                               \
+      (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top, Nout, K, out, kind, limit, alpha);
+    if (tm == 64) {
+      const int gy = (Nout + 127) / 128;
+      if (gated) { XGM_GG(true, 4, 2, false, gy) } else { XGM_GG(false, 4, 2, false, gy) }
+    } else {
+      const int gy = (Nout + 31) / 32;
+      if (gated) { XGM_GG(true, 1, 2, true, gy) } else { XGM_GG(false, 1, 2, true, gy) }
+    }
+#undef XGM_GG
     return 0;
   }
-  dim3 grid(tiles, (Nout + 63) / 64);
+  dim3 grid(cap / 16, (Nout + 63) / 64);
   if (gated) {
     XGM_DISPATCH_T(f32, grouped_gemm_kernel<T, true><<<grid, 256, 0, st>>>((const T*)A, lda, (const T*)Wt, rows, tile_expert,
-                                                                            top, Nout, K, out, kind, limit, alpha);)
+                                                                            tm, top, Nout, K, out, kind, limit, alpha);)
   } else {
     XGM_DISPATCH_T(f32, grouped_gemm_kernel<T, false><<<grid, 256, 0, st>>>((const T*)A, lda, (const T*)Wt, rows,
-                                                                             tile_expert, top, Nout, K, out, kind, limit,
-                                                                             alpha);)
+                                                                             tile_expert, tm, top, Nout, K, out, kind,
+                                                                             limit, alpha);)
   }
   return 0;
 }

@@ -20,13 +20,16 @@ void qk_norm_cache(const void*, bool, int64_t, int, int, int, const float*, cons
 int masked_attention(const void*, bool, const void*, const void*, const int32_t*, int, int, const int32_t*,
                      const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, float,
                      hipStream_t);
+int masked_attention_mfma(const void*, const void*, const void*, const int32_t*, int, int, const int32_t*, const int32_t*,
+                          const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, int, int,
+                          float, hipStream_t);
 int ssm_scan(const void*, bool, int64_t, const void*, int64_t, const float*, const float*, const float*, float*,
              const int32_t*, const int32_t*, const int32_t*, float*, int, int, int, int, int, hipStream_t);
 void gated_group_norm(const float*, const void*, bool, int64_t, const float*, float, void*, int, int, int, hipStream_t);
 void glu_act(const void*, bool, int64_t, void*, int, int, int, float, float, hipStream_t);
 int grouped_router(const float*, const float*, int, int, int, int, int, float, int32_t*, float*, hipStream_t);
-int moe_align(const int32_t*, int, int, int, int32_t*, int32_t*, int32_t*, hipStream_t);
-int grouped_gemm(const void*, bool, int64_t, const void*, const int32_t*, const int32_t*, int, int, int, int, bool, void*,
+int moe_align(const int32_t*, int, int, int, int, int32_t*, int32_t*, int32_t*, hipStream_t);
+int grouped_gemm(const void*, bool, int64_t, const void*, const int32_t*, const int32_t*, int, int, int, int, int, bool, void*,
                  int, float, float, bool, hipStream_t);
 void moe_combine(const float*, const int32_t*, const float*, int, int, int, float*, hipStream_t);
 void canon_conv(const float*, const float*, float*, const int32_t*, const int32_t*, const int32_t*, void*, bool, int, int,
@@ -102,6 +105,17 @@ PYBIND11_MODULE(_mixers, m) {
                                    P<const float>(sink), P<void>(out), T, H, G, dk, dv, mask, size, scale, S(st));
     check(rc, "masked_attention");
   });
+  m.def("masked_attention_mfma", [](uintptr_t q, uintptr_t kc, uintptr_t vc, uintptr_t bt, int bt_width, int bs,
+                                    uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t temp, uintptr_t sink,
+                                    uintptr_t out, int T, int ns, int max_q, int H, int G, int dk, int dv, int mask,
+                                    int size, float scale, uintptr_t st) {
+    if (bs < 1 || bt_width < 1) throw std::invalid_argument("masked_attention_mfma: inconsistent sizes");
+    int rc = xgm::masked_attention_mfma(P<const void>(q), P<const void>(kc), P<const void>(vc), P<const int32_t>(bt),
+                                        bt_width, bs, P<const int32_t>(qsl), P<const int32_t>(sl), P<const int32_t>(slots),
+                                        P<const float>(temp), P<const float>(sink), P<void>(out), T, ns, max_q, H, G, dk,
+                                        dv, mask, size, scale, S(st));
+    check(rc, "masked_attention_mfma");
+  });
   m.def("ssm_scan", [](uintptr_t xbc, bool f32, int64_t ld_x, uintptr_t dt, int64_t ld_dt, uintptr_t dt_bias,
                        uintptr_t A_log, uintptr_t D, uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots,
                        uintptr_t y, int ns, int H, int G, int N, int Pd, uintptr_t st) {
@@ -131,18 +145,18 @@ PYBIND11_MODULE(_mixers, m) {
                                  P<int32_t>(ids), P<float>(wts), S(st));
     check(rc, "grouped_router");
   });
-  m.def("moe_align", [](uintptr_t ids, int pairs, int E, int cap, uintptr_t rows, uintptr_t tile_expert, uintptr_t dest,
-                        uintptr_t st) {
-    int rc = xgm::moe_align(P<const int32_t>(ids), pairs, E, cap, P<int32_t>(rows), P<int32_t>(tile_expert),
+  m.def("moe_align", [](uintptr_t ids, int pairs, int E, int cap, int tm, uintptr_t rows, uintptr_t tile_expert,
+                        uintptr_t dest, uintptr_t st) {
+    int rc = xgm::moe_align(P<const int32_t>(ids), pairs, E, cap, tm, P<int32_t>(rows), P<int32_t>(tile_expert),
                             P<int32_t>(dest), S(st));
     check(rc, "moe_align");
   });
   m.def("grouped_gemm", [](uintptr_t A, bool f32, int64_t lda, uintptr_t Wt, uintptr_t rows, uintptr_t tile_expert, int cap,
-                           int top, int Nout, int K, bool gated, uintptr_t out, int kind, float limit, float alpha,
+                           int tm, int top, int Nout, int K, bool gated, uintptr_t out, int kind, float limit, float alpha,
                            bool mfma, uintptr_t st) {
     if (top < 1 || lda < K) throw std::invalid_argument("grouped_gemm: inconsistent sizes");
     int rc = xgm::grouped_gemm(P<const void>(A), f32, lda, P<const void>(Wt), P<const int32_t>(rows),
-                               P<const int32_t>(tile_expert), cap, top, Nout, K, gated, P<void>(out), kind, limit, alpha,
+                               P<const int32_t>(tile_expert), cap, tm, top, Nout, K, gated, P<void>(out), kind, limit, alpha,
                                mfma, S(st));
     check(rc, "grouped_gemm");
   });
@@ -150,7 +164,7 @@ PYBIND11_MODULE(_mixers, m) {
     xgm::moe_combine(P<const float>(y), P<const int32_t>(dest), P<const float>(wts), T, top, W, P<float>(out), S(st));
     check(0, "moe_combine");
   });
-  m.attr("MOE_TILE_M") = 16;
+
   m.def("canon_conv", [](uintptr_t x, uintptr_t w, uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots,
                          uintptr_t out, bool out_f32, int ns, int max_q, int W, int taps, uintptr_t st) {
     if (taps < 1 || taps > 8) throw std::invalid_argument("canon_conv: taps must be in [1, 8]");

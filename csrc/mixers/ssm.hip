@@ -10,35 +10,37 @@
 //   gated_group_norm  v = y * silu(z);  each of `ng` equal parts of v divided by its own root mean
 //                     square, times w: the gate comes BEFORE the norm.
 //
-// One wave = 16 state columns x 4 row slices: lane (p = lane & 15, qn = lane >> 4) owns rows
-// [qn * NI, (qn + 1) * NI) of column p in registers. B / C / x / dt of 16 tokens at a time are
-// staged in LDS; the per-token work is 2 FMAs per owned state element plus a 4-lane sum.
+// One workgroup = (sequence, head, 64 state columns), 4 waves: lane p owns column p, wave w owns rows
+// [w * NI, (w + 1) * NI) of it in registers (state rows are read and written 256 bytes at a time). B / C / x /
+// dt of TT tokens at a time are staged in LDS (two buffers: the next tile's global loads are issued before the
+// current tile's steps and stored after them). Per token a wave does 2 FMAs per owned state element; the four
+// waves' partial sums of y meet in LDS once per tile.
 #include "mixers_common.h"
 
 namespace xgm {
 
-constexpr int kScanCols = 16;   // state columns per wave
-constexpr int kScanTile = 16;   // tokens staged per LDS tile
+constexpr int kScanCols = 64;   // state columns per workgroup
 
-template <typename T, int NI>
-__global__ __launch_bounds__(64) void ssm_scan_kernel(const T* __restrict__ xbc, int64_t ld_x, const T* __restrict__ dt_raw,
-                                                      int64_t ld_dt, const float* __restrict__ dt_bias,
-                                                      const float* __restrict__ A_log, const float* __restrict__ Dskip,
-                                                      float* __restrict__ state, const int32_t* __restrict__ qsl,
-                                                      const int32_t* __restrict__ seq_lens,
-                                                      const int32_t* __restrict__ slots, float* __restrict__ y, int H, int G,
-                                                      int N, int P) {
-  constexpr int LDN = 4 * (NI + 4);  // padded row of B or C: slice qn starts at qn * (NI + 4)
-  __shared__ __attribute__((aligned(16))) float Bs[kScanTile][LDN];
-  __shared__ __attribute__((aligned(16))) float Cs[kScanTile][LDN];
-  __shared__ float xs[kScanTile][kScanCols];
-  __shared__ float dts[kScanTile], decs[kScanTile];
+template <typename T, int NI, int TT>
+__global__ __launch_bounds__(256) void ssm_scan_kernel(const T* __restrict__ xbc, int64_t ld_x, const T* __restrict__ dt_raw,
+                                                       int64_t ld_dt, const float* __restrict__ dt_bias,
+                                                       const float* __restrict__ A_log, const float* __restrict__ Dskip,
+                                                       float* __restrict__ state, const int32_t* __restrict__ qsl,
+                                                       const int32_t* __restrict__ seq_lens,
+                                                       const int32_t* __restrict__ slots, float* __restrict__ y, int H,
+                                                       int G, int N, int P) {
+  constexpr int NB = 4 * NI;                 // padded state rows
+  constexpr int ROW = 2 * NB + kScanCols;    // staged floats per token: [B | C | x]
+  constexpr int PER = (TT * ROW + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float stage[2][TT][ROW];
+  __shared__ float dts[2][TT], decs[2][TT];
+  __shared__ float ypart[TT][4][kScanCols];
   const int s = blockIdx.x, h = blockIdx.y;
   const int q0 = qsl[s], q = qsl[s + 1] - q0, slot = slots[s];
   if (slot < 0 || q <= 0) return;
   const int ctx = seq_lens[s] - q;
-  const int lane = threadIdx.x, pl = lane & 15, qn = lane >> 4;
-  const int p = blockIdx.z * kScanCols + pl;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int p0 = blockIdx.z * kScanCols, p = p0 + lane;
   const bool pok = p < P;
   const int g = h / (H / G);
   const int inner = H * P;
@@ -47,46 +49,78 @@ __global__ __launch_bounds__(64) void ssm_scan_kernel(const T* __restrict__ xbc,
   float S[NI];
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
-    const int n = qn * NI + i;
+    const int n = wave * NI + i;
     S[i] = (ctx > 0 && pok && n < N) ? Sg[(int64_t)n * P + p] : 0.f;
   }
-  for (int t0 = 0; t0 < q; t0 += kScanTile) {
-    const int nt = min(kScanTile, q - t0);
-    __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
-      const T* row = xbc + (int64_t)(q0 + t0 + tt) * ld_x;
-      for (int n = lane; n < 4 * NI; n += 64) {
-        const int qq = n / NI, ii = n % NI;
-        Bs[tt][qq * (NI + 4) + ii] = n < N ? ldf(row + inner + g * N + n) : 0.f;
-        Cs[tt][qq * (NI + 4) + ii] = n < N ? ldf(row + inner + G * N + g * N + n) : 0.f;
+  float pre[PER], pre_dt = 0.f;
+  auto fetch = [&](int t0) {  // global loads of the tile starting at token t0 (zeros past the end / the sizes)
+    const int nt = min(TT, q - t0);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = threadIdx.x + 256 * j;
+      const int tt = e / ROW, c = e % ROW;
+      float v = 0.f;
+      if (tt < nt) {
+        const T* row = xbc + (int64_t)(q0 + t0 + tt) * ld_x;
+        if (c < NB) {
+          if (c < N) v = ldf(row + inner + g * N + c);
+        } else if (c < 2 * NB) {
+          if (c - NB < N) v = ldf(row + inner + G * N + g * N + (c - NB));
+        } else if (p0 + c - 2 * NB < P) {
+          v = ldf(row + h * P + p0 + c - 2 * NB);
+        }
       }
-      if (lane < kScanCols) xs[tt][lane] = (blockIdx.z * kScanCols + lane < P) ? ldf(row + h * P + blockIdx.z * kScanCols + lane) : 0.f;
+      pre[j] = v;
     }
-    if (lane < nt) {
-      const float d = softplusf(ldf(dt_raw + (int64_t)(q0 + t0 + lane) * ld_dt + h) + bias);
-      dts[lane] = d;
-      decs[lane] = expf(-rate * d);
+    if (threadIdx.x < nt) pre_dt = ldf(dt_raw + (int64_t)(q0 + t0 + threadIdx.x) * ld_dt + h);
+  };
+  auto commit = [&](int buf, int t0) {
+    const int nt = min(TT, q - t0);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = threadIdx.x + 256 * j;
+      if (e < TT * ROW) (&stage[buf][0][0])[e] = pre[j];
     }
-    __syncthreads();
+    if (threadIdx.x < nt) {
+      const float d = softplusf(pre_dt + bias);
+      dts[buf][threadIdx.x] = d;
+      decs[buf][threadIdx.x] = expf(-rate * d);
+    }
+  };
+  fetch(0);
+  commit(0, 0);
+  __syncthreads();
+  int buf = 0;
+  for (int t0 = 0; t0 < q; t0 += TT, buf ^= 1) {
+    const int nt = min(TT, q - t0);
+    const bool more = t0 + TT < q;
+    if (more) fetch(t0 + TT);
     for (int tt = 0; tt < nt; ++tt) {
-      const float a = decs[tt], xv = xs[tt][pl], dx = dts[tt] * xv;
-      const float* Br = &Bs[tt][qn * (NI + 4)];
-      const float* Cr = &Cs[tt][qn * (NI + 4)];
+      const float* Br = &stage[buf][tt][wave * NI];
+      const float* Cr = &stage[buf][tt][NB + wave * NI];
+      const float a = decs[buf][tt], dx = dts[buf][tt] * stage[buf][tt][2 * NB + lane];
       float acc = 0.f;
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         S[i] = a * S[i] + dx * Br[i];
         acc += S[i] * Cr[i];
       }
-      acc += __shfl_xor(acc, 16, 64);
-      acc += __shfl_xor(acc, 32, 64);
-      if (qn == 0 && pok) y[(int64_t)(q0 + t0 + tt) * inner + h * P + p] = acc + dsk * xv;
+      ypart[tt][wave][lane] = acc;
     }
+    __syncthreads();
+    for (int e = threadIdx.x; e < nt * kScanCols; e += 256) {
+      const int tt = e / kScanCols, c = e % kScanCols;
+      if (p0 + c < P)
+        y[(int64_t)(q0 + t0 + tt) * inner + h * P + p0 + c] =
+            ypart[tt][0][c] + ypart[tt][1][c] + ypart[tt][2][c] + ypart[tt][3][c] + dsk * stage[buf][tt][2 * NB + c];
+    }
+    if (more) commit(buf ^ 1, t0 + TT);
+    __syncthreads();
   }
   if (pok) {
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      const int n = qn * NI + i;
+      const int n = wave * NI + i;
       if (n < N) Sg[(int64_t)n * P + p] = S[i];
     }
   }
@@ -117,16 +151,16 @@ int ssm_scan(const void* xbc, bool f32, int64_t ld_x, const void* dt_raw, int64_
   if (ns <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G != 0 || N < 1 || N > 256 || P < 1) return -1;
   dim3 grid(ns, H, (P + kScanCols - 1) / kScanCols);
-#define XGM_SS(NI)                                                                                                       \
-  XGM_DISPATCH_T(f32, ssm_scan_kernel<T, NI><<<grid, 64, 0, st>>>((const T*)xbc, ld_x, (const T*)dt_raw, ld_dt, dt_bias, \
-                                                                   A_log, Dskip, state, qsl, seq_lens, slots, y, H, G, N, \
-                                                                   P);)                                                   \
+#define XGM_SS(NI, TT)                                                                                                 \
+  XGM_DISPATCH_T(f32, ssm_scan_kernel<T, NI, TT><<<grid, 256, 0, st>>>((const T*)xbc, ld_x, (const T*)dt_raw, ld_dt,  \
+                                                                        dt_bias, A_log, Dskip, state, qsl, seq_lens,  \
+                                                                        slots, y, H, G, N, P);)                       \
   return 0;
-  if (N <= 16) { XGM_SS(4) }
-  if (N <= 32) { XGM_SS(8) }
-  if (N <= 64) { XGM_SS(16) }
-  if (N <= 128) { XGM_SS(32) }
-  XGM_SS(64)
+  if (N <= 16) { XGM_SS(4, 16) }
+  if (N <= 32) { XGM_SS(8, 16) }
+  if (N <= 64) { XGM_SS(16, 16) }
+  if (N <= 128) { XGM_SS(32, 16) }
+  XGM_SS(64, 8)
 #undef XGM_SS
 }
 

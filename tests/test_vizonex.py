@@ -556,7 +556,8 @@ def test_router_groups_correction_and_weights(device, E, count, keep, top):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-@pytest.mark.parametrize("W,ff,E,top,T", [(40, 24, 6, 3, 50), (64, 32, 16, 2, 300), (96, 80, 3, 1, 7), (64, 16, 40, 4, 1)])
+@pytest.mark.parametrize("W,ff,E,top,T", [(40, 24, 6, 3, 50), (64, 32, 16, 2, 300), (96, 80, 3, 1, 7), (64, 16, 40, 4, 1),
+                                          (64, 48, 4, 2, 200), (128, 64, 2, 2, 333)])
 def test_experts_weighted_sum(device, dtype, W, ff, E, top, T):
     from xgserve.models.vizonex import GroupedRouterMoE
     td = getattr(torch, dtype)

@@ -471,8 +471,9 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         assert q.is_contiguous() and kcache.is_contiguous() and vcache.is_contiguous()
         assert kcache.dtype == vcache.dtype == q.dtype
         bt = _i32(sm.block_tables)
-        if (ATTN_MFMA and q.dtype == torch.bfloat16 and hasattr(mixers(), "masked_attention_mfma")
-                and dk % 32 == 0 and dv % 16 == 0 and dk <= 256 and dv <= 256):
+        if ATTN_MFMA and q.dtype == torch.bfloat16 and sm.max_q > 1 and dk % 32 == 0 and dv % 16 == 0 and dk <= 128 \
+                and dv <= 128:
+            # prompt portions (also beside single tokens): 16 tokens x one head per wave on the matrix cores
             mixers().masked_attention_mfma(q.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), bt.data_ptr(), bt.shape[1],
                                            block_size, _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
                                            _i32(sm.slots).data_ptr(), _p(temp), _p(sink), out.data_ptr(), T, sm.num_seqs,
@@ -561,6 +562,7 @@ def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, eps: flo
 GLU_GELU_TANH, GLU_CLAMPED = 0, 1
 # XGS_TUNE moe_mfma=0: the general grouped GEMM for bf16 too (A/B and tests)
 MOE_MFMA = tune.get_bool("moe_mfma", True)
+MOE_TILE_SMALL, MOE_TILE_BIG = 16, 64   # rows per expert tile of the sorted layout
 
 
 def _glu_ref(g, u, kind, limit, alpha):
@@ -630,19 +632,20 @@ def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: to
             out.index_add_(0, tt, (a @ w2[e].float().t()) * wts[tt, jj][:, None])
         return out
     M = mixers()
-    tm = M.MOE_TILE_M
     assert h.is_contiguous() and w13.is_contiguous() and w2.is_contiguous() and w13.dtype == w2.dtype == h.dtype
     pairs = T * top
+    # rows of an expert are padded to whole tiles: 64-row tiles once the average expert has that many, else 16
+    tm = MOE_TILE_BIG if pairs >= MOE_TILE_BIG * E else MOE_TILE_SMALL
     cap = (pairs + E * (tm - 1) + tm - 1) // tm * tm
     dev = h.device
     meta = torch.empty(cap + cap // tm + pairs, dtype=torch.int32, device=dev)
     rows, tile_e, dest = meta[:cap], meta[cap:cap + cap // tm], meta[cap + cap // tm:]
-    M.moe_align(_i32(ids).data_ptr(), pairs, E, cap, rows.data_ptr(), tile_e.data_ptr(), dest.data_ptr(), stream_ptr())
+    M.moe_align(_i32(ids).data_ptr(), pairs, E, cap, tm, rows.data_ptr(), tile_e.data_ptr(), dest.data_ptr(), stream_ptr())
     act = torch.empty(cap, F_, dtype=h.dtype, device=dev)
-    M.grouped_gemm(h.data_ptr(), is_f32(h), h.stride(0), w13.data_ptr(), rows.data_ptr(), tile_e.data_ptr(), cap, top, F_,
-                   K, True, act.data_ptr(), int(kind), float(limit), float(alpha), MOE_MFMA, stream_ptr())
+    M.grouped_gemm(h.data_ptr(), is_f32(h), h.stride(0), w13.data_ptr(), rows.data_ptr(), tile_e.data_ptr(), cap, tm, top,
+                   F_, K, True, act.data_ptr(), int(kind), float(limit), float(alpha), MOE_MFMA, stream_ptr())
     y = torch.empty(cap, W, dtype=torch.float32, device=dev)
-    M.grouped_gemm(act.data_ptr(), is_f32(act), F_, w2.data_ptr(), rows.data_ptr(), tile_e.data_ptr(), cap, top, W, F_,
+    M.grouped_gemm(act.data_ptr(), is_f32(act), F_, w2.data_ptr(), rows.data_ptr(), tile_e.data_ptr(), cap, tm, top, W, F_,
                    False, y.data_ptr(), 0, 0.0, 0.0, MOE_MFMA, stream_ptr())
     out = torch.empty(T, W, dtype=torch.float32, device=dev)
     M.moe_combine(y.data_ptr(), dest.data_ptr(), wts.data_ptr(), T, top, W, out.data_ptr(), stream_ptr())
