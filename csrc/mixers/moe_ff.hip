@@ -321,6 +321,85 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __re
     }
 }
 
+// ---- prompt-sized steps (layout tiles of 64 rows): a workgroup owns 64 rows x 4 x 16 NT columns. The A rows
+// (gathered token rows, shared by the four waves) go through LDS, 32 k at a time in two buffers, one barrier
+// per step; every wave streams its own B columns from global memory.
+template <bool GATED, int NT>
+__global__ __launch_bounds__(256) void grouped_gemm_mfma_lds_kernel(const bf16* __restrict__ A, int64_t lda,
+                                                                    const bf16* __restrict__ Wt,
+                                                                    const int32_t* __restrict__ rows,
+                                                                    const int32_t* __restrict__ tile_expert, int top,
+                                                                    int Nout, int K, void* __restrict__ out, int kind,
+                                                                    float limit, float alpha) {
+  constexpr int MT = 4, LDA = 40, NG = GATED ? NT : 1;
+  __shared__ __attribute__((aligned(16))) uint16_t As[2][64 * LDA];
+  const int tile = blockIdx.x;
+  const int e = tile_expert[tile];
+  if (e < 0) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = (blockIdx.y * 4 + wave) * 16 * NT;
+  const int l16 = lane & 15, kg = lane >> 4;
+  const int64_t wrows = GATED ? 2 * (int64_t)Nout : (int64_t)Nout;
+  const bf16* We = Wt + (int64_t)e * wrows * K;
+  const int rbase = tile * 64;
+  // staging: thread -> (row = tid / 4, 16-byte chunk = tid % 4) of the 64 x 32 A block
+  const int srow = threadIdx.x >> 2, sch = threadIdx.x & 3;
+  const int pa = rows[rbase + srow];
+  const bf16* asrc = A + (int64_t)(GATED ? max(pa, 0) / top : rbase + srow) * lda + sch * 8;
+  f32x4_t acc[MT][NT], accu[MT][NG];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < NG; ++j) accu[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  xgk::st16(&As[0][srow * LDA + sch * 8], pa >= 0 ? ld16(asrc) : make_uint4(0, 0, 0, 0));
+  __syncthreads();
+  int buf = 0;
+  const bool wave_on = n0 < Nout;
+  for (int k0 = 0; k0 < K; k0 += 32, buf ^= 1) {
+    const bool more = k0 + 32 < K;
+    uint4 anext = make_uint4(0, 0, 0, 0);
+    if (more && pa >= 0) anext = ld16(asrc + k0 + 32);
+    if (wave_on) {
+      uint4 bv[NT], uv[NG];
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const int n = min(n0 + 16 * j, Nout - 16) + l16;  // whole 16-column tiles; clamped ones are not stored
+        bv[j] = ld16(We + (int64_t)n * K + k0 + kg * 8);
+        if (GATED) uv[j] = ld16(We + (int64_t)(Nout + n) * K + k0 + kg * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const uint4 av = ld16(&As[buf][(16 * i + l16) * LDA + kg * 8]);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          acc[i][j] = mfma16x16x32(as_frag(av), as_frag(bv[j]), acc[i][j]);
+          if (GATED) accu[i][j] = mfma16x16x32(as_frag(av), as_frag(uv[j]), accu[i][j]);
+        }
+      }
+    }
+    if (more) xgk::st16(&As[buf ^ 1][srow * LDA + sch * 8], anext);
+    __syncthreads();
+  }
+  if (!wave_on) return;
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int n = n0 + 16 * j + l16;
+      if (n0 + 16 * j >= Nout) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int rr = rbase + 16 * i + kg * 4 + r;
+        if (rows[rr] < 0) continue;
+        if (GATED) ((bf16*)out)[(int64_t)rr * Nout + n] = f2bf(glu(kind, acc[i][j][r], accu[i][GATED ? j : 0][r], limit, alpha));
+        else ((float*)out)[(int64_t)rr * Nout + n] = acc[i][j][r];
+      }
+    }
+}
+
 __global__ void moe_combine_kernel(const float* __restrict__ y, const int32_t* __restrict__ dest,
                                    const float* __restrict__ wts, int top, int W, float* __restrict__ out) {
   const int t = blockIdx.x;
@@ -367,9 +446,13 @@ int grouped_gemm(const void* A, bool f32, int64_t lda, const void* Wt, const int
 #define XGM_GG(GATED, MT, NT, SPLITK, GY)                                                                            \
   grouped_gemm_mfma_kernel<GATED, MT, NT, SPLITK><<<dim3(cap / tm, GY), 256, 0, st>>>(                               \
       (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top, Nout, K, out, kind, limit, alpha);
-    if (tm == 64) {
-      const int gy = (Nout + 127) / 128;
-      if (gated) { XGM_GG(true, 4, 2, false, gy) } else { XGM_GG(false, 4, 2, false, gy) }
+    if (tm == 64) {  // gated: 64 x 128 per workgroup (two accumulator sets); plain: 64 x 256
+      if (gated)
+        grouped_gemm_mfma_lds_kernel<true, 2><<<dim3(cap / 64, (Nout + 127) / 128), 256, 0, st>>>(
+            (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top, Nout, K, out, kind, limit, alpha);
+      else
+        grouped_gemm_mfma_lds_kernel<false, 4><<<dim3(cap / 64, (Nout + 255) / 256), 256, 0, st>>>(
+            (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top, Nout, K, out, kind, limit, alpha);
     } else {
       const int gy = (Nout + 31) / 32;
       if (gated) { XGM_GG(true, 1, 2, true, gy) } else { XGM_GG(false, 1, 2, true, gy) }

@@ -10,31 +10,33 @@
 //   gated_group_norm  v = y * silu(z);  each of `ng` equal parts of v divided by its own root mean
 //                     square, times w: the gate comes BEFORE the norm.
 //
-// One workgroup = (sequence, head, 64 state columns), 4 waves: lane p owns column p, wave w owns rows
+// One workgroup = (sequence, head, 64 state columns), NW waves: lane p owns column p, wave w owns rows
 // [w * NI, (w + 1) * NI) of it in registers (state rows are read and written 256 bytes at a time). B / C / x /
 // dt of TT tokens at a time are staged in LDS (two buffers: the next tile's global loads are issued before the
-// current tile's steps and stored after them). Per token a wave does 2 FMAs per owned state element; the four
-// waves' partial sums of y meet in LDS once per tile.
+// current tile's steps and stored after them). Per token a wave does 2 FMAs per owned state element; the
+// waves' partial sums of y meet in LDS once per tile. Eight waves (two per SIMD) hide the LDS and dependency
+// latency of the serial token loop.
 #include "mixers_common.h"
 
 namespace xgm {
 
 constexpr int kScanCols = 64;   // state columns per workgroup
 
-template <typename T, int NI, int TT>
-__global__ __launch_bounds__(256) void ssm_scan_kernel(const T* __restrict__ xbc, int64_t ld_x, const T* __restrict__ dt_raw,
+template <typename T, int NI, int TT, int NW>
+__global__ __launch_bounds__(64 * NW) void ssm_scan_kernel(const T* __restrict__ xbc, int64_t ld_x, const T* __restrict__ dt_raw,
                                                        int64_t ld_dt, const float* __restrict__ dt_bias,
                                                        const float* __restrict__ A_log, const float* __restrict__ Dskip,
                                                        float* __restrict__ state, const int32_t* __restrict__ qsl,
                                                        const int32_t* __restrict__ seq_lens,
                                                        const int32_t* __restrict__ slots, float* __restrict__ y, int H,
                                                        int G, int N, int P) {
-  constexpr int NB = 4 * NI;                 // padded state rows
+  constexpr int NB = NW * NI;                // padded state rows
+  constexpr int NTH = 64 * NW;
   constexpr int ROW = 2 * NB + kScanCols;    // staged floats per token: [B | C | x]
-  constexpr int PER = (TT * ROW + 255) / 256;
+  constexpr int PER = (TT * ROW + NTH - 1) / NTH;
   __shared__ __attribute__((aligned(16))) float stage[2][TT][ROW];
   __shared__ float dts[2][TT], decs[2][TT];
-  __shared__ float ypart[TT][4][kScanCols];
+  __shared__ float ypart[TT][NW][kScanCols];
   const int s = blockIdx.x, h = blockIdx.y;
   const int q0 = qsl[s], q = qsl[s + 1] - q0, slot = slots[s];
   if (slot < 0 || q <= 0) return;
@@ -57,7 +59,7 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const T* __restrict__ xbc
     const int nt = min(TT, q - t0);
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      const int e = threadIdx.x + 256 * j;
+      const int e = threadIdx.x + NTH * j;
       const int tt = e / ROW, c = e % ROW;
       float v = 0.f;
       if (tt < nt) {
@@ -78,7 +80,7 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const T* __restrict__ xbc
     const int nt = min(TT, q - t0);
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      const int e = threadIdx.x + 256 * j;
+      const int e = threadIdx.x + NTH * j;
       if (e < TT * ROW) (&stage[buf][0][0])[e] = pre[j];
     }
     if (threadIdx.x < nt) {
@@ -108,11 +110,14 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const T* __restrict__ xbc
       ypart[tt][wave][lane] = acc;
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < nt * kScanCols; e += 256) {
+    for (int e = threadIdx.x; e < nt * kScanCols; e += NTH) {
       const int tt = e / kScanCols, c = e % kScanCols;
-      if (p0 + c < P)
-        y[(int64_t)(q0 + t0 + tt) * inner + h * P + p0 + c] =
-            ypart[tt][0][c] + ypart[tt][1][c] + ypart[tt][2][c] + ypart[tt][3][c] + dsk * stage[buf][tt][2 * NB + c];
+      if (p0 + c < P) {
+        float v = dsk * stage[buf][tt][2 * NB + c];
+#pragma unroll
+        for (int w = 0; w < NW; ++w) v += ypart[tt][w][c];
+        y[(int64_t)(q0 + t0 + tt) * inner + h * P + p0 + c] = v;
+      }
     }
     if (more) commit(buf ^ 1, t0 + TT);
     __syncthreads();
@@ -151,16 +156,16 @@ int ssm_scan(const void* xbc, bool f32, int64_t ld_x, const void* dt_raw, int64_
   if (ns <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G != 0 || N < 1 || N > 256 || P < 1) return -1;
   dim3 grid(ns, H, (P + kScanCols - 1) / kScanCols);
-#define XGM_SS(NI, TT)                                                                                                 \
-  XGM_DISPATCH_T(f32, ssm_scan_kernel<T, NI, TT><<<grid, 256, 0, st>>>((const T*)xbc, ld_x, (const T*)dt_raw, ld_dt,  \
-                                                                        dt_bias, A_log, Dskip, state, qsl, seq_lens,  \
-                                                                        slots, y, H, G, N, P);)                       \
+#define XGM_SS(NI, TT, NW)                                                                                           \
+  XGM_DISPATCH_T(f32, ssm_scan_kernel<T, NI, TT, NW><<<grid, 64 * NW, 0, st>>>((const T*)xbc, ld_x, (const T*)dt_raw, \
+                                                                                ld_dt, dt_bias, A_log, Dskip, state,  \
+                                                                                qsl, seq_lens, slots, y, H, G, N, P);) \
   return 0;
-  if (N <= 16) { XGM_SS(4, 16) }
-  if (N <= 32) { XGM_SS(8, 16) }
-  if (N <= 64) { XGM_SS(16, 16) }
-  if (N <= 128) { XGM_SS(32, 16) }
-  XGM_SS(64, 8)
+  if (N <= 16) { XGM_SS(4, 16, 4) }
+  if (N <= 32) { XGM_SS(8, 16, 4) }
+  if (N <= 64) { XGM_SS(8, 8, 8) }
+  if (N <= 128) { XGM_SS(16, 8, 8) }
+  XGM_SS(32, 8, 8)
 #undef XGM_SS
 }
 
