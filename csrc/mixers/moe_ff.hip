@@ -209,17 +209,18 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const T* __restrict__
 }
 
 // ---- matrix-core form (bf16; K % 32 == 0, Nout % 16 == 0). A / B fragments come straight from global
-// memory (16 bytes per lane), accumulators are fp32. Two shapes of one kernel:
-//   SPLITK = false (prompt-sized steps, layout tiles of 64 rows): a workgroup owns 16 MT rows x 4 x 16 NT columns,
-//            each wave 16 NT of the columns over the whole K;
-//   SPLITK = true  (few rows per expert, layout tiles of 16 rows): a workgroup owns 16 rows x 16 NT columns, its four
-//            waves a quarter of K each (short dependent load chains, 4 x the workgroups); the partial sums meet in LDS.
+// memory (16 or 32 bytes per lane and step), accumulators are fp32. For steps with few rows per expert (layout
+// tiles of 16 rows). Two shapes of one kernel:
+//   SPLITK = false: a workgroup owns 16 MT rows x 4 x 16 NT columns, each wave 16 NT of the columns over the whole K
+//            (a long loop, four steps' loads in flight);
+//   SPLITK = true:  a workgroup owns 16 rows x 16 NT columns, its four waves a quarter of K each; the partial sums
+//            meet in LDS.
 using xgk::as_frag;
 using xgk::f32x4_t;
 using xgk::ld16;
 using xgk::mfma16x16x32;
 
-template <bool GATED, int MT, int NT, bool SPLITK>
+template <bool GATED, int MT, int NT, bool SPLITK, bool K64>
 __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __restrict__ A, int64_t lda,
                                                                 const bf16* __restrict__ Wt,
                                                                 const int32_t* __restrict__ rows,
@@ -244,7 +245,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __re
   for (int i = 0; i < MT; ++i) {
     const int pa = rows[rbase + 16 * i + l16];
     aok[i] = pa >= 0;
-    arow[i] = A + (int64_t)(GATED ? max(pa, 0) / top : rbase + 16 * i + l16) * lda + kg * 8;
+    arow[i] = A + (int64_t)(GATED ? max(pa, 0) / top : rbase + 16 * i + l16) * lda + kg * (K64 ? 16 : 8);
   }
   f32x4_t acc[MT][NT], accu[MT][NG];
 #pragma unroll
@@ -254,27 +255,38 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __re
 #pragma unroll
     for (int j = 0; j < NG; ++j) accu[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
-  const int kper = SPLITK ? ((K / 32 + 3) / 4) * 32 : K;
+  // K64: a lane takes 32 contiguous bytes of a row per step (the four lanes of a row 128 bytes) and feeds them
+  // to two MFMAs. A and B use the same assignment of k to (lane, MFMA), and a sum over k has no order.
+  constexpr int KS = K64 ? 64 : 32, KL = K64 ? 16 : 8;
+  const int kper = SPLITK ? ((K / KS + 3) / 4) * KS : K;
   const int kbeg = SPLITK ? wave * kper : 0, kend = min(K, kbeg + kper);
-#pragma unroll 2
-  for (int k0 = kbeg; k0 < kend; k0 += 32) {
-    uint4 av[MT], bv[NT], uv[NG];
+#pragma unroll(SPLITK ? 2 : 4)
+  for (int k0 = kbeg; k0 < kend; k0 += KS) {
+    uint4 av[MT][K64 ? 2 : 1], bv[NT][K64 ? 2 : 1], uv[NG][K64 ? 2 : 1];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) av[i] = aok[i] ? ld16(arow[i] + k0) : make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int h = 0; h < (K64 ? 2 : 1); ++h)
+        av[i][h] = aok[i] ? ld16(arow[i] + k0 + 8 * h) : make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       const int n = min(n0 + 16 * j, Nout - 16) + l16;  // whole 16-column tiles (Nout % 16 == 0); clamped ones are not stored
-      bv[j] = ld16(We + (int64_t)n * K + k0 + kg * 8);
-      if (GATED) uv[j] = ld16(We + (int64_t)(Nout + n) * K + k0 + kg * 8);
+#pragma unroll
+      for (int h = 0; h < (K64 ? 2 : 1); ++h) {
+        bv[j][h] = ld16(We + (int64_t)n * K + k0 + kg * KL + 8 * h);
+        if (GATED) uv[j][h] = ld16(We + (int64_t)(Nout + n) * K + k0 + kg * KL + 8 * h);
+      }
     }
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        // D = A (rows x k) B (k x cols): accumulator entry r of lane (l16, kg) is row kg * 4 + r, column l16
-        acc[i][j] = mfma16x16x32(as_frag(av[i]), as_frag(bv[j]), acc[i][j]);
-        if (GATED) accu[i][j] = mfma16x16x32(as_frag(av[i]), as_frag(uv[j]), accu[i][j]);
-      }
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int h = 0; h < (K64 ? 2 : 1); ++h) {
+          // D = A (rows x k) B (k x cols): accumulator entry r of lane (l16, kg) is row kg * 4 + r, column l16
+          acc[i][j] = mfma16x16x32(as_frag(av[i][h]), as_frag(bv[j][h]), acc[i][j]);
+          if (GATED) accu[i][j] = mfma16x16x32(as_frag(av[i][h]), as_frag(uv[j][h]), accu[i][j]);
+        }
   }
   if (SPLITK) {  // MT == 1: waves 1..3 hand their partial sums to wave 0
     if (wave > 0) {
@@ -321,31 +333,36 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __re
     }
 }
 
-// ---- prompt-sized steps (layout tiles of 64 rows): a workgroup owns 64 rows x 4 x 16 NT columns. The A rows
+// ---- prompt-sized steps (layout tiles of 64 or 128 rows): a workgroup owns 16 MT rows x 4 x 16 NT columns. The A rows
 // (gathered token rows, shared by the four waves) go through LDS, 32 k at a time in two buffers, one barrier
-// per step; every wave streams its own B columns from global memory.
-template <bool GATED, int NT>
+// per step; every wave streams its own B columns from global memory into registers.
+template <bool GATED, int MT, int NT>
 __global__ __launch_bounds__(256) void grouped_gemm_mfma_lds_kernel(const bf16* __restrict__ A, int64_t lda,
                                                                     const bf16* __restrict__ Wt,
                                                                     const int32_t* __restrict__ rows,
-                                                                    const int32_t* __restrict__ tile_expert, int top,
-                                                                    int Nout, int K, void* __restrict__ out, int kind,
-                                                                    float limit, float alpha) {
-  constexpr int MT = 4, LDA = 40, NG = GATED ? NT : 1;
-  __shared__ __attribute__((aligned(16))) uint16_t As[2][64 * LDA];
-  const int tile = blockIdx.x;
-  const int e = tile_expert[tile];
+                                                                    const int32_t* __restrict__ tile_expert, int tm,
+                                                                    int top, int Nout, int K, void* __restrict__ out,
+                                                                    int kind, float limit, float alpha) {
+  constexpr int LDA = 40, NG = GATED ? NT : 1, RPT = MT / 4;  // RPT: staged rows per thread
+  __shared__ __attribute__((aligned(16))) uint16_t As[2][16 * MT * LDA];
+  const int tile = blockIdx.x;  // 16 MT rows of a layout tile of tm rows
+  const int e = tile_expert[tile * 16 * MT / tm];
   if (e < 0) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n0 = (blockIdx.y * 4 + wave) * 16 * NT;
   const int l16 = lane & 15, kg = lane >> 4;
   const int64_t wrows = GATED ? 2 * (int64_t)Nout : (int64_t)Nout;
   const bf16* We = Wt + (int64_t)e * wrows * K;
-  const int rbase = tile * 64;
-  // staging: thread -> (row = tid / 4, 16-byte chunk = tid % 4) of the 64 x 32 A block
+  const int rbase = tile * 16 * MT;
+  // staging: thread -> (rows tid / 4 + 64 r, 16-byte chunk = tid % 4) of the (16 MT) x 32 A block
   const int srow = threadIdx.x >> 2, sch = threadIdx.x & 3;
-  const int pa = rows[rbase + srow];
-  const bf16* asrc = A + (int64_t)(GATED ? max(pa, 0) / top : rbase + srow) * lda + sch * 8;
+  int pa[RPT];
+  const bf16* asrc[RPT];
+#pragma unroll
+  for (int r = 0; r < RPT; ++r) {
+    pa[r] = rows[rbase + srow + 64 * r];
+    asrc[r] = A + (int64_t)(GATED ? max(pa[r], 0) / top : rbase + srow + 64 * r) * lda + sch * 8;
+  }
   f32x4_t acc[MT][NT], accu[MT][NG];
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
@@ -354,14 +371,17 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_lds_kernel(const bf16* 
 #pragma unroll
     for (int j = 0; j < NG; ++j) accu[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
-  xgk::st16(&As[0][srow * LDA + sch * 8], pa >= 0 ? ld16(asrc) : make_uint4(0, 0, 0, 0));
+#pragma unroll
+  for (int r = 0; r < RPT; ++r)
+    xgk::st16(&As[0][(srow + 64 * r) * LDA + sch * 8], pa[r] >= 0 ? ld16(asrc[r]) : make_uint4(0, 0, 0, 0));
   __syncthreads();
   int buf = 0;
   const bool wave_on = n0 < Nout;
   for (int k0 = 0; k0 < K; k0 += 32, buf ^= 1) {
     const bool more = k0 + 32 < K;
-    uint4 anext = make_uint4(0, 0, 0, 0);
-    if (more && pa >= 0) anext = ld16(asrc + k0 + 32);
+    uint4 anext[RPT];
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) anext[r] = (more && pa[r] >= 0) ? ld16(asrc[r] + k0 + 32) : make_uint4(0, 0, 0, 0);
     if (wave_on) {
       uint4 bv[NT], uv[NG];
 #pragma unroll
@@ -376,11 +396,14 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_lds_kernel(const bf16* 
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
           acc[i][j] = mfma16x16x32(as_frag(av), as_frag(bv[j]), acc[i][j]);
-          if (GATED) accu[i][j] = mfma16x16x32(as_frag(av), as_frag(uv[j]), accu[i][j]);
+          if (GATED) accu[i][j] = mfma16x16x32(as_frag(av), as_frag(uv[GATED ? j : 0]), accu[i][GATED ? j : 0]);
         }
       }
     }
-    if (more) xgk::st16(&As[buf ^ 1][srow * LDA + sch * 8], anext);
+    if (more) {
+#pragma unroll
+      for (int r = 0; r < RPT; ++r) xgk::st16(&As[buf ^ 1][(srow + 64 * r) * LDA + sch * 8], anext[r]);
+    }
     __syncthreads();
   }
   if (!wave_on) return;
@@ -441,22 +464,24 @@ int grouped_gemm(const void* A, bool f32, int64_t lda, const void* Wt, const int
                  int cap, int tm, int top, int Nout, int K, bool gated, void* out, int kind, float limit, float alpha,
                  bool mfma, hipStream_t st) {
   if (cap <= 0) return 0;
-  if ((tm != 16 && tm != 64) || cap % tm != 0 || Nout < 1 || K < 1) return -1;
+  if ((tm != 16 && tm != 64 && tm != 128) || cap % tm != 0 || Nout < 1 || K < 1) return -1;
   if (!f32 && mfma && K % 32 == 0 && Nout % 16 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)Wt % 16 == 0) {
-#define XGM_GG(GATED, MT, NT, SPLITK, GY)                                                                            \
-  grouped_gemm_mfma_kernel<GATED, MT, NT, SPLITK><<<dim3(cap / tm, GY), 256, 0, st>>>(                               \
+#define XGM_GG(GATED, K64)                                                                                          \
+  grouped_gemm_mfma_kernel<GATED, 1, 2, true, K64><<<dim3(cap / tm, (Nout + 31) / 32), 256, 0, st>>>(                \
       (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top, Nout, K, out, kind, limit, alpha);
-    if (tm == 64) {  // gated: 64 x 128 per workgroup (two accumulator sets); plain: 64 x 256
-      if (gated)
-        grouped_gemm_mfma_lds_kernel<true, 2><<<dim3(cap / 64, (Nout + 127) / 128), 256, 0, st>>>(
-            (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top, Nout, K, out, kind, limit, alpha);
-      else
-        grouped_gemm_mfma_lds_kernel<false, 4><<<dim3(cap / 64, (Nout + 255) / 256), 256, 0, st>>>(
-            (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top, Nout, K, out, kind, limit, alpha);
+#define XGM_GL(GATED, MT, NT)                                                                                         \
+  grouped_gemm_mfma_lds_kernel<GATED, MT, NT><<<dim3(cap / (16 * MT), (Nout + 64 * NT - 1) / (64 * NT)), 256, 0, st>>>( \
+      (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, tm, top, Nout, K, out, kind, limit, alpha);
+    if (tm == 128) {         // gated: 64 x 128 per workgroup (two accumulator sets); plain: 128 x 128
+      if (gated) { XGM_GL(true, 4, 2) } else { XGM_GL(false, 8, 2) }
+    } else if (tm == 64) {   // gated: 64 x 128; plain: 64 x 256
+      if (gated) { XGM_GL(true, 4, 2) } else { XGM_GL(false, 4, 4) }
+    } else if (K % 64 == 0) {
+      if (gated) { XGM_GG(true, true) } else { XGM_GG(false, true) }
     } else {
-      const int gy = (Nout + 31) / 32;
-      if (gated) { XGM_GG(true, 1, 2, true, gy) } else { XGM_GG(false, 1, 2, true, gy) }
+      if (gated) { XGM_GG(true, false) } else { XGM_GG(false, false) }
     }
+#undef XGM_GL
 #undef XGM_GG
     return 0;
   }

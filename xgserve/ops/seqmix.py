@@ -562,7 +562,7 @@ def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, eps: flo
 GLU_GELU_TANH, GLU_CLAMPED = 0, 1
 # XGS_TUNE moe_mfma=0: the general grouped GEMM for bf16 too (A/B and tests)
 MOE_MFMA = tune.get_bool("moe_mfma", True)
-MOE_TILE_SMALL, MOE_TILE_BIG = 16, 64   # rows per expert tile of the sorted layout
+MOE_TILE_SMALL, MOE_TILES_BIG = 16, (128, 64)   # rows per expert tile of the sorted layout
 
 
 def _glu_ref(g, u, kind, limit, alpha):
@@ -634,8 +634,8 @@ def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: to
     M = mixers()
     assert h.is_contiguous() and w13.is_contiguous() and w2.is_contiguous() and w13.dtype == w2.dtype == h.dtype
     pairs = T * top
-    # rows of an expert are padded to whole tiles: 64-row tiles once the average expert has that many, else 16
-    tm = MOE_TILE_BIG if pairs >= MOE_TILE_BIG * E else MOE_TILE_SMALL
+    # rows of an expert are padded to whole tiles: 128 / 64-row tiles once the average expert has that many, else 16
+    tm = next((t for t in MOE_TILES_BIG if pairs >= t * E), MOE_TILE_SMALL)
     cap = (pairs + E * (tm - 1) + tm - 1) // tm * tm
     dev = h.device
     meta = torch.empty(cap + cap // tm + pairs, dtype=torch.int32, device=dev)
