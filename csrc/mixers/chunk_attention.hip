@@ -221,21 +221,46 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
   // the sink starts the running softmax: weight exp(sink - m) = 1 with no value behind it
   float m = sink ? sink[head] : -INFINITY, l = sink ? 1.f : 0.f;
 
+  // staging: thread -> (row = tid / 4, 16-byte chunks tid % 4, + 4, ..) of the K row and of the V row. The next
+  // tile's rows are loaded into registers before the current tile's products and stored after them.
   const int srow = threadIdx.x >> 2, squad = threadIdx.x & 3;
-  for (int k0 = kmin; k0 <= pos_last; k0 += kKT) {
-    __syncthreads();
-    {
-      const int kabs = k0 + srow;
-      const bool ok = kabs <= pos_last;
-      const int64_t row = ok ? (int64_t)bt[kabs / bs] * bs + kabs % bs : 0;
-      const bf16* ks = kcache + (row * G + g) * dk;
-      const bf16* vs = vcache + (row * G + g) * dv;
-      for (int ch = squad; ch * 8 < dk; ch += 4)
-        xgk::st16(ktile + srow * LDK + ch * 8, ok ? xgk::ld16(ks + ch * 8) : make_uint4(0, 0, 0, 0));
-      for (int ch = squad; ch * 8 < dv; ch += 4)
-        xgk::st16(vtile + srow * LDV + ch * 8, ok ? xgk::ld16(vs + ch * 8) : make_uint4(0, 0, 0, 0));
+  constexpr int NVC = (NMT_MAX + 1) / 2;
+  uint4 sk[NKK_MAX], sv[NVC];
+  auto fetch = [&](int k0) {
+    const int kabs = k0 + srow;
+    const bool ok = kabs <= pos_last;
+    const int64_t row = ok ? (int64_t)bt[kabs / bs] * bs + kabs % bs : 0;
+    const bf16* ks = kcache + (row * G + g) * dk;
+    const bf16* vs = vcache + (row * G + g) * dv;
+#pragma unroll
+    for (int it = 0; it < NKK_MAX; ++it) {
+      const int ch = squad + 4 * it;
+      sk[it] = (ok && ch * 8 < dk) ? xgk::ld16(ks + ch * 8) : make_uint4(0, 0, 0, 0);
     }
+#pragma unroll
+    for (int it = 0; it < NVC; ++it) {
+      const int ch = squad + 4 * it;
+      sv[it] = (ok && ch * 8 < dv) ? xgk::ld16(vs + ch * 8) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int it = 0; it < NKK_MAX; ++it) {
+      const int ch = squad + 4 * it;
+      if (ch * 8 < dk) xgk::st16(ktile + srow * LDK + ch * 8, sk[it]);
+    }
+#pragma unroll
+    for (int it = 0; it < NVC; ++it) {
+      const int ch = squad + 4 * it;
+      if (ch * 8 < dv) xgk::st16(vtile + srow * LDV + ch * 8, sv[it]);
+    }
+  };
+  if (kmin <= pos_last) fetch(kmin);
+  for (int k0 = kmin; k0 <= pos_last; k0 += kKT) {
+    __syncthreads();  // the previous tile is consumed
+    commit();
     __syncthreads();
+    if (k0 + kKT <= pos_last) fetch(k0 + kKT);
     if (!wave_on) continue;
     xgk::f32x4_t sacc[4];
 #pragma unroll
