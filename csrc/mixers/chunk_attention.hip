@@ -164,9 +164,10 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
 
 
 // ------------------------------------------------------------------ matrix-core form (bf16, dk % 32 == 0, dv % 16 == 0)
-// A wave owns 16 query slots: 16 consecutive tokens of one sequence x one query head. The 4 waves of a
-// workgroup are RH query heads of one key/value head x 4 / RH token tiles, so a tile of 64 keys (K rows and
-// V rows, staged once in LDS) serves all of them. S^T = K Q^T on v_mfma_f32_16x16x32_bf16: the accumulator
+// A wave owns 16 query slots. Prompt portions: 16 consecutive tokens of one sequence x one query head; the 4 waves
+// of a workgroup are RH query heads of one key/value head x 4 / RH token tiles, so a tile of 64 keys (K rows and
+// V rows, staged once in LDS) serves all of them. Steps of single tokens: the slots are the (up to 64) query heads
+// of one key/value head at the sequence's one token, one workgroup per (sequence, key/value head). S^T = K Q^T on v_mfma_f32_16x16x32_bf16: the accumulator
 // holds, per lane, 16 keys of ONE slot, and packed to bf16 it is the B operand of O^T += V^T P^T, whose A
 // operand (V^T) is a transposed LDS read of the staged V rows.
 constexpr int kKT = 64;
@@ -177,34 +178,47 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
     const int32_t* __restrict__ block_tables, int bt_width, int bs, const int32_t* __restrict__ qsl,
     const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots, const float* __restrict__ temp,
     const float* __restrict__ sink, bf16* __restrict__ out, int H, int G, int dk, int dv, int mask, int size, float scale,
-    int RH) {
+    int RH, int head_slots, float* __restrict__ part_o, float* __restrict__ part_ml, int Ttot) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   const int LDK = dk + 8, LDV = dv + 8;
   uint16_t* ktile = lds;                 // [kKT][LDK]
   uint16_t* vtile = lds + kKT * LDK;     // [kKT][LDV]
   const int s = blockIdx.z;
   const int q0 = qsl[s], qn = qsl[s + 1] - q0;
-  if (slots[s] < 0 || qn <= 0) return;
-  const int tpb = 4 / RH;                // token tiles per workgroup
-  const int t0 = blockIdx.x * 16 * tpb;
-  if (t0 >= qn) return;
   const int rep = H / G;
-  const int hblocks = (rep + RH - 1) / RH;
-  const int g = blockIdx.y / hblocks, hb = blockIdx.y % hblocks;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int li = lane & 15, kg = lane >> 4;
-  const int hr = hb * RH + wave % RH;                // head within the group
-  const int tok = t0 + (wave / RH) * 16 + li;        // this lane's slot: token within the sequence's rows
-  const bool wave_on = hr < rep && t0 + (wave / RH) * 16 < qn;
-  const bool valid = wave_on && tok < qn;
+  if (slots[s] < 0 || qn <= 0) {
+    // a padding row of a single-token step still gets a defined output row
+    if (head_slots && qn == 1)
+      for (int d = threadIdx.x; d < rep * dv; d += blockDim.x) out[((int64_t)q0 * H + blockIdx.y * rep) * dv + d] = 0;
+    return;
+  }
+  // prompt portions: slots = 16 tokens of one head; single-token steps (head_slots): slots = 16 heads of the token
+  const int tpb = head_slots ? 1 : 4 / RH;  // token tiles per workgroup
+  const int t0 = head_slots ? 0 : blockIdx.x * 16 * tpb;
+  if (t0 >= qn) return;
+  const int hblocks = (rep + RH - 1) / RH;
+  const int g = head_slots ? blockIdx.y : blockIdx.y / hblocks, hb = blockIdx.y % hblocks;
+  const int hr = head_slots ? wave * 16 + li : hb * RH + wave % RH;   // head within the group
+  const int tok = head_slots ? 0 : t0 + (wave / RH) * 16 + li;         // token within the sequence's rows
+  const bool wave_on = head_slots ? wave * 16 < rep : (hr < rep && t0 + (wave / RH) * 16 < qn);
+  const bool valid = wave_on && hr < rep && tok < qn;
   const int head = g * rep + min(hr, rep - 1);
   const int ctx = seq_lens[s] - qn;
   const int pos_q = ctx + min(tok, qn - 1);
   const int lo_q = first_visible(mask, size, pos_q);
   const int nkk = dk / 32, nmt = dv / 16;
   // keys any slot of this workgroup can see
-  const int kmin = first_visible(mask, size, ctx + t0);
-  const int pos_last = ctx + min(qn, t0 + 16 * tpb) - 1;
+  int kmin = first_visible(mask, size, ctx + t0);
+  int pos_last = ctx + (head_slots ? 1 : min(qn, t0 + 16 * tpb)) - 1;
+  // single-token steps divide the visible key tiles over gridDim.x workgroups (merged by a second launch)
+  const int nsplit = head_slots ? gridDim.x : 1;
+  if (nsplit > 1) {
+    const int tiles = (pos_last - kmin + kKT) / kKT, per = (tiles + nsplit - 1) / nsplit;
+    kmin += blockIdx.x * per * kKT;
+    pos_last = min(pos_last, kmin + per * kKT - 1);  // may leave this share empty
+  }
   const int32_t* bt = block_tables + (int64_t)s * bt_width;
 
   xgk::bf16x8_t qf[NKK_MAX];
@@ -219,7 +233,8 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
 #pragma unroll
   for (int mt = 0; mt < NMT_MAX; ++mt) o[mt] = xgk::f32x4_t{0.f, 0.f, 0.f, 0.f};
   // the sink starts the running softmax: weight exp(sink - m) = 1 with no value behind it
-  float m = sink ? sink[head] : -INFINITY, l = sink ? 1.f : 0.f;
+  const bool with_sink = sink && (nsplit == 1 || blockIdx.x == 0);  // the sink counts once: in the first share
+  float m = with_sink ? sink[head] : -INFINITY, l = with_sink ? 1.f : 0.f;
 
   // staging: thread -> (row = tid / 4, 16-byte chunks tid % 4, + 4, ..) of the K row and of the V row. The next
   // tile's rows are loaded into registers before the current tile's products and stored after them.
@@ -325,7 +340,17 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
         }
     }
   }
-  if (valid) {
+  if (valid && nsplit > 1) {  // unnormalised share: (m, l) and the weighted value sum
+    const int64_t row = ((int64_t)blockIdx.x * Ttot + q0 + tok) * H + head;
+    if (kg == 0) {
+      part_ml[2 * row] = m;
+      part_ml[2 * row + 1] = l;
+    }
+#pragma unroll
+    for (int mt = 0; mt < NMT_MAX; ++mt)
+      if (mt < nmt)
+        *reinterpret_cast<float4*>(part_o + row * dv + mt * 16 + 4 * kg) = make_float4(o[mt][0], o[mt][1], o[mt][2], o[mt][3]);
+  } else if (valid) {
     const float inv = l > 0.f ? 1.f / l : 0.f;
     bf16* op = out + ((int64_t)(q0 + tok) * H + head) * dv;
 #pragma unroll
@@ -336,6 +361,32 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
         w.y = xgk::pack2(o[mt][2] * inv, o[mt][3] * inv);
         *reinterpret_cast<uint2*>(op + mt * 16 + 4 * kg) = w;
       }
+  }
+}
+
+// merge the key shares of a single-token step: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s
+__global__ void masked_attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                const int32_t* __restrict__ slots, bf16* __restrict__ out, int Ttot, int H,
+                                                int dv, int nsplit) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  if (slots[t] < 0) return;  // single-token steps: row t is sequence t (its output row was zeroed)
+  float M = -INFINITY;
+  for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, part_ml[2 * (((int64_t)sp * Ttot + t) * H + h)]);
+  float L = 0.f;
+  for (int sp = 0; sp < nsplit; ++sp) {
+    const int64_t row = ((int64_t)sp * Ttot + t) * H + h;
+    const float ms = part_ml[2 * row];
+    if (ms != -INFINITY) L += __expf(ms - M) * part_ml[2 * row + 1];
+  }
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  for (int d = threadIdx.x; d < dv; d += blockDim.x) {
+    float acc = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) {
+      const int64_t row = ((int64_t)sp * Ttot + t) * H + h;
+      const float ms = part_ml[2 * row];
+      if (ms != -INFINITY) acc += __expf(ms - M) * part_o[row * dv + d];
+    }
+    out[((int64_t)t * H + h) * dv + d] = f2bf(acc * inv);
   }
 }
 
@@ -387,7 +438,7 @@ int masked_attention(const void* q, bool f32, const void* kcache, const void* vc
 int masked_attention_mfma(const void* q, const void* kcache, const void* vcache, const int32_t* block_tables, int bt_width,
                           int bs, const int32_t* qsl, const int32_t* seq_lens, const int32_t* slots, const float* temp,
                           const float* sink, void* out, int T_, int ns, int max_q, int H, int G, int dk, int dv, int mask,
-                          int size, float scale, hipStream_t st) {
+                          int size, float scale, int nsplit, float* part_o, float* part_ml, hipStream_t st) {
   if (T_ <= 0 || ns <= 0 || max_q <= 0) return 0;
   if (G <= 0 || H % G != 0 || dk % 32 != 0 || dv % 16 != 0 || dk > 128 || dv > 128 || mask < 0 || mask > 2 ||
       (mask != kMaskCausal && size < 1))
@@ -395,13 +446,21 @@ int masked_attention_mfma(const void* q, const void* kcache, const void* vcache,
   const int rep = H / G;
   const int RH = rep >= 4 ? 4 : rep >= 2 ? 2 : 1;
   const int tpb = 4 / RH;
+  // a step of single tokens: one workgroup per (sequence, key/value head), its query heads as the slots
+  const int head_slots = (max_q == 1 && T_ == ns) ? 1 : 0;
+  if (head_slots && rep > 64) return -3;
   dim3 grid((max_q + 16 * tpb - 1) / (16 * tpb), G * ((rep + RH - 1) / RH), ns);
+  if (!head_slots || nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) nsplit = 1;
+  if (head_slots) grid = dim3(nsplit, G, ns);
   const size_t lds = (size_t)kKT * (dk + 8 + dv + 8) * sizeof(uint16_t);
 #define XGM_MM(NKK, NMT)                                                                                              \
   masked_attention_mfma_kernel<NKK, NMT><<<grid, 256, lds, st>>>((const bf16*)q, (const bf16*)kcache,                 \
                                                                  (const bf16*)vcache, block_tables, bt_width, bs, qsl, \
                                                                  seq_lens, slots, temp, sink, (bf16*)out, H, G, dk, dv, \
-                                                                 mask, size, scale, RH);                               \
+                                                                 mask, size, scale, RH, head_slots, part_o, part_ml,   \
+                                                                 T_);                                                  \
+  if (nsplit > 1)                                                                                                     \
+    masked_attention_combine_kernel<<<dim3(T_, H), 64, 0, st>>>(part_o, part_ml, slots, (bf16*)out, T_, H, dv, nsplit); \
   return 0;
   if (dk <= 64 && dv <= 64) { XGM_MM(2, 4) }
   if (dk <= 128 && dv <= 128) { XGM_MM(4, 8) }

@@ -22,7 +22,7 @@ int masked_attention(const void*, bool, const void*, const void*, const int32_t*
                      hipStream_t);
 int masked_attention_mfma(const void*, const void*, const void*, const int32_t*, int, int, const int32_t*, const int32_t*,
                           const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, int, int,
-                          float, hipStream_t);
+                          float, int, float*, float*, hipStream_t);
 int ssm_scan(const void*, bool, int64_t, const void*, int64_t, const float*, const float*, const float*, float*,
              const int32_t*, const int32_t*, const int32_t*, float*, int, int, int, int, int, hipStream_t);
 void gated_group_norm(const float*, const void*, bool, int64_t, const float*, float, void*, int, int, int, hipStream_t);
@@ -108,12 +108,13 @@ PYBIND11_MODULE(_mixers, m) {
   m.def("masked_attention_mfma", [](uintptr_t q, uintptr_t kc, uintptr_t vc, uintptr_t bt, int bt_width, int bs,
                                     uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t temp, uintptr_t sink,
                                     uintptr_t out, int T, int ns, int max_q, int H, int G, int dk, int dv, int mask,
-                                    int size, float scale, uintptr_t st) {
-    if (bs < 1 || bt_width < 1) throw std::invalid_argument("masked_attention_mfma: inconsistent sizes");
+                                    int size, float scale, int nsplit, uintptr_t part_o, uintptr_t part_ml,
+                                    uintptr_t st) {
+    if (bs < 1 || bt_width < 1 || nsplit < 1) throw std::invalid_argument("masked_attention_mfma: inconsistent sizes");
     int rc = xgm::masked_attention_mfma(P<const void>(q), P<const void>(kc), P<const void>(vc), P<const int32_t>(bt),
                                         bt_width, bs, P<const int32_t>(qsl), P<const int32_t>(sl), P<const int32_t>(slots),
                                         P<const float>(temp), P<const float>(sink), P<void>(out), T, ns, max_q, H, G, dk,
-                                        dv, mask, size, scale, S(st));
+                                        dv, mask, size, scale, nsplit, P<float>(part_o), P<float>(part_ml), S(st));
     check(rc, "masked_attention_mfma");
   });
   m.def("ssm_scan", [](uintptr_t xbc, bool f32, int64_t ld_x, uintptr_t dt, int64_t ld_dt, uintptr_t dt_bias,

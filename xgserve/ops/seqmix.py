@@ -420,6 +420,8 @@ def residual_norm(x: torch.Tensor, y1: Optional[torch.Tensor], a1: Optional[torc
 MASK_CAUSAL, MASK_WINDOW, MASK_CHUNK = 0, 1, 2
 # XGS_TUNE attn_mfma=0: the general (any size, fp32-capable) kernel for bf16 too (A/B and tests)
 ATTN_MFMA = tune.get_bool("attn_mfma", True)
+ATTN_MAX_SPLITS = 8      # key shares per single-token row, at most
+ATTN_SPLIT_WGS = 2048    # ... while the launch stays under about this many workgroups
 
 
 def first_visible(mask: int, size: int, pos: int) -> int:
@@ -471,13 +473,23 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         assert q.is_contiguous() and kcache.is_contiguous() and vcache.is_contiguous()
         assert kcache.dtype == vcache.dtype == q.dtype
         bt = _i32(sm.block_tables)
-        if ATTN_MFMA and q.dtype == torch.bfloat16 and sm.max_q > 1 and dk % 32 == 0 and dv % 16 == 0 and dk <= 128 \
-                and dv <= 128:
-            # prompt portions (also beside single tokens): 16 tokens x one head per wave on the matrix cores
+        single = sm.max_q == 1 and T == sm.num_seqs
+        if ATTN_MFMA and q.dtype == torch.bfloat16 and dk % 32 == 0 and dv % 16 == 0 and dk <= 128 and dv <= 128 \
+                and (not single or H // G <= 64):
+            # matrix cores: prompt portions (also beside single tokens) as 16 tokens x one head per wave, steps of
+            # single tokens as the query heads of one key/value head per wave
+            nsplit, part_o, part_ml = 1, None, None
+            if single:  # divide the visible key tiles over several workgroups (merged by a second launch)
+                tiles = (size + 63) // 64 if mask != MASK_CAUSAL else ATTN_MAX_SPLITS
+                nsplit = max(1, min(ATTN_MAX_SPLITS, tiles, ATTN_SPLIT_WGS // max(1, T * G)))
+                if nsplit > 1:
+                    part_o = torch.empty(nsplit * T * H * dv, dtype=torch.float32, device=q.device)
+                    part_ml = torch.empty(nsplit * T * H * 2, dtype=torch.float32, device=q.device)
             mixers().masked_attention_mfma(q.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), bt.data_ptr(), bt.shape[1],
                                            block_size, _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
                                            _i32(sm.slots).data_ptr(), _p(temp), _p(sink), out.data_ptr(), T, sm.num_seqs,
-                                           sm.max_q, H, G, dk, dv, int(mask), int(size), float(scale), stream_ptr())
+                                           sm.max_q, H, G, dk, dv, int(mask), int(size), float(scale), nsplit,
+                                           _p(part_o), _p(part_ml), stream_ptr())
             return out
         mixers().masked_attention(q.data_ptr(), is_f32(q), kcache.data_ptr(), vcache.data_ptr(), bt.data_ptr(),
                                   bt.shape[1], block_size, _i32(sm.positions).data_ptr(), _i32(sm.token_seq).data_ptr(),
