@@ -233,7 +233,7 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
 #pragma unroll
   for (int mt = 0; mt < NMT_MAX; ++mt) o[mt] = xgk::f32x4_t{0.f, 0.f, 0.f, 0.f};
   // the sink starts the running softmax: weight exp(sink - m) = 1 with no value behind it
-  const bool with_sink = sink && (nsplit == 1 || blockIdx.x == 0);  // the sink counts once: in the first share
+  const bool with_sink = sink && (nsplit == 1 || blockIdx.x == 0);  // the sink enters the first share only
   float m = with_sink ? sink[head] : -INFINITY, l = with_sink ? 1.f : 0.f;
 
   // staging: thread -> (row = tid / 4, 16-byte chunks tid % 4, + 4, ..) of the K row and of the V row. The next

@@ -3,10 +3,11 @@
 //   glu_act          [gate | up] rows -> act(gate) * up':
 //                      kGluGeluTanh   0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * u
 //                      kGluClamped    g' = min(g, limit), u' = clamp(u, -limit, limit):  g' sigmoid(alpha g') (u' + 1)
-//   grouped_router   fp32 router logits -> sigmoid scores; choice scores = score + correction; experts form
-//                    `count` equal groups of neighbours, a group scores the sum of its two largest choice
-//                    scores, only experts of the best `keep` groups can be chosen (the others count as
-//                    -inf); the `top` largest choice scores win; weights = score (WITHOUT correction) * scale
+//   grouped_router   fp32 router logits -> sigmoid scores; selection score = score + correction; the experts are
+//                    split into `count` contiguous groups of equal size, a group is rated by the sum of its two
+//                    highest selection scores, members of the `keep` highest-rated groups stay eligible (all
+//                    others are excluded outright: selection score -inf); the `top` highest eligible selection
+//                    scores win; weight = score * scale (the correction does not enter it, no normalisation)
 //   moe_align        (token, choice) pairs sorted by expert into tiles of `tm` rows (padded with -1)
 //   grouped_gemm     per tile: rows x expert weights; first GEMM with the gated activation fused,
 //                    second GEMM to fp32 rows

@@ -2,13 +2,13 @@
 // carried per sequence slot, and the gated group norm that follows it.
 //
 //   ssm_scan          per head h (group g = h / (H / G)), state S [N x P] fp32 per (slot, head):
-//                       dt_t = softplus(dt_raw_t + dt_bias_h)            (no clamp)
+//                       dt_t = softplus(dt_raw_t + dt_bias_h)            (not limited to a range)
 //                       S_t  = exp(-exp(A_log_h) dt_t) S_(t-1) + dt_t B_t x_t^T
 //                       y_t  = S_t^T C_t + D_h x_t
 //                     x / B / C are columns of one activation row [x (H P) | B (G N) | C (G N)] (already
 //                     through their short convolution and activation), dt_raw a column block of another.
 //   gated_group_norm  v = y * silu(z);  each of `ng` equal parts of v divided by its own root mean
-//                     square, times w: the gate comes BEFORE the norm.
+//                     square, times w (gated first, normed second).
 //
 // One workgroup = (sequence, head, 64 state columns), NW waves: lane p owns column p, wave w owns rows
 // [w * NI, (w + 1) * NI) of it in registers (state rows are read and written 256 bytes at a time). B / C / x /

@@ -513,7 +513,7 @@ def test_state_space_mixer_over_portions_and_slots(device, H, P, N, G, ng, taps)
 
 
 @pytest.mark.parametrize("device", OP_CASES)
-def test_gate_comes_before_the_group_norm(device):
+def test_group_norm_of_the_gated_output(device):
     g = torch.Generator().manual_seed(2)
     y, z, w = torch.randn(5, 48, generator=g), torch.randn(5, 60, generator=g), torch.randn(48, generator=g)
     for ng in (1, 3, 48):
@@ -540,8 +540,9 @@ def test_gated_activations_and_their_clamps(device):
 @pytest.mark.parametrize("E,count,keep,top", [(16, 4, 3, 2), (6, 3, 2, 3), (5, 5, 2, 2), (4, 1, 1, 1), (72, 8, 3, 6),
                                               (160, 4, 1, 8)])
 def test_router_groups_correction_and_weights(device, E, count, keep, top):
-    """Strongly negative corrections make every choice score negative: an expert outside the kept groups must
-    count as -inf, not 0. The weights carry no correction and are not renormalised."""
+    """Strongly negative corrections make every selection score negative, so an expert outside the eligible
+    groups has to be excluded outright (scoring it 0 would let it win). The weights are the plain scores times
+    the scale."""
     g = torch.Generator().manual_seed(E)
     z = torch.randn(40, E, generator=g) * 2
     corr = torch.randn(E, generator=g) * 0.5 - 3.0

@@ -17,7 +17,7 @@ Mixers (reusable modules, every constant a parameter):
     head (a sink: no key, no value).
   * `SelectiveStateSpace` ("mamba2"): input projection [z | x | B | C | dt], a short convolution +
     silu over [x | B | C], a scalar-decay state-space recurrence on an fp32 [state x vdim] state per
-    head and slot, gate silu(z) BEFORE a group RMS norm, output projection.
+    head and slot, gating by silu(z) followed by a group RMS norm, output projection.
 Feed-forward: `GatedMLP` (gelu-tanh gate) or `GroupedRouterMoE` (sigmoid router with a selection-only
 correction and group-limited top-k over clamped-GLU experts, plus an always-on shared expert).
 

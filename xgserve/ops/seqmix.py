@@ -522,7 +522,7 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
 def ssm_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, A_log: torch.Tensor, D: torch.Tensor,
              state: torch.Tensor, H: int, G: int, N: int, P: int, sm: SeqMeta) -> torch.Tensor:
     """Per head h (group h // (H / G)), with x / B / C the column blocks [H P | G N | G N] of `xbc` and
-    dt = softplus(dt_raw + dt_bias) (no clamp):  S <- exp(-exp(A_log_h) dt) S + dt B x^T  (S is N x P),
+    dt = softplus(dt_raw + dt_bias) (not limited to a range):  S <- exp(-exp(A_log_h) dt) S + dt B x^T  (S is N x P),
     y = S^T C + D_h x. state fp32 [slots, H, N, P] is carried and updated. Returns y fp32 [T, H * P]."""
     T = xbc.shape[0]
     y = torch.empty(T, H * P, dtype=torch.float32, device=xbc.device)
@@ -603,9 +603,10 @@ def glu_act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.702
 def grouped_router(logits: torch.Tensor, correction: Optional[torch.Tensor], count: int, keep: int, top: int,
                    scale: float):
     """fp32 router logits [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]). Scores are
-    sigmoid(logits); experts are CHOSEN by score + correction, restricted to the `keep` best of `count`
-    groups of neighbouring experts (a group scores the sum of its two largest choice scores; experts of
-    other groups count as -inf), and WEIGHTED by score * scale (no correction, no renormalisation)."""
+    sigmoid(logits). Selection uses score + correction: the experts form `count` contiguous groups of equal
+    size, a group is rated by the sum of its two highest selection scores, and only members of the `keep`
+    highest-rated groups are eligible (everything else is excluded outright, selection score -inf). The
+    returned weights are score * scale: the correction does not enter them and they are not normalised."""
     T, E = logits.shape
     if not native_device(logits):
         s = torch.sigmoid(logits.float())
