@@ -453,6 +453,14 @@ def test_attention_chunk_edges_pages_and_far_keys(device, dtype, shape, size, bs
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("shape", [(40, 2, 32, 16), (3, 1, 128, 128)], ids=["rep20", "d128"])
+def test_attention_many_heads_per_key_head_and_large_heads(device, dtype, shape):
+    """More query heads per key/value head than one wave's 16 slots; the largest matrix-core head size."""
+    H, G, dk, dv = shape
+    _attention_case(device, dtype, H, G, dk, dv, 96, 16, 150, 100)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
 def test_attention_without_sink_and_sink_alone(device, dtype):
     _attention_case(device, dtype, 4, 2, 32, 16, 16, 4, 70, 40, use_sink=False)
     # a huge sink takes all the weight: the output vanishes
